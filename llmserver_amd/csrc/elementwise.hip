@@ -290,6 +290,37 @@ LSA_EXPORT int lsa_swiglu(int dtype, const void* gate_up, void* out, int n_token
     return dtype ? launch_swiglu<bf16_t, 0>(gate_up, out, n_tokens, inter, stream)
                  : launch_swiglu<float, 0>(gate_up, out, n_tokens, inter, stream);
 }
+
+// Ungated activation, where the numbers lie: x = act(x); act 0: silu, 1: the tanh form of GELU, 2: max(x, 0)^2.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ x, long n, int activation) {
+    const long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * V;
+    if (i >= n) return;
+    auto act = [&](float z) {
+        if (activation == 2) { const float r = fmaxf(z, 0.f); return r * r; }
+        return activation == 1 ? gate_activation<1>(z) : gate_activation<0>(z);
+    };
+    if (V > 1) {
+        Vec16<T> a = load_vec16(x + i);
+#pragma unroll
+        for (int k = 0; k < V; ++k) a.v[k] = (T)act((float)a.v[k]);
+        store_vec16(x + i, a);
+    } else {
+        x[i] = (T)act((float)x[i]);
+    }
+}
+LSA_EXPORT int lsa_activation(int dtype, void* x, long n, int activation, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (activation < 0 || activation > 2) return -1;
+#define LSA_LAUNCH(T) do { \
+        constexpr int V = Elem<T>::kVec; \
+        if (n % V == 0) activation_kernel<T, V><<<(unsigned)((n / V + 255) / 256), 256, 0, stream>>>((T*)x, n, activation); \
+        else activation_kernel<T, 1><<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((T*)x, n, activation); \
+    } while (0)
+    if (dtype) LSA_LAUNCH(bf16_t); else LSA_LAUNCH(float);
+#undef LSA_LAUNCH
+    LSA_LAUNCH_CHECK();
+}
 LSA_EXPORT int lsa_add_bias(int dtype, void* y, const float* bias, int n_tokens, int n, hipStream_t stream) {
     return dtype ? launch_add_bias<bf16_t>(y, bias, n_tokens, n, stream)
                  : launch_add_bias<float>(y, bias, n_tokens, n, stream);

@@ -101,7 +101,8 @@ __global__ void latent_prepare_kernel(
 template <typename T>
 __global__ void gate_heads_kernel(const T* __restrict__ y, const T* __restrict__ mixed, const T* __restrict__ up_values,
                                   int rank, int row_width, const T* __restrict__ proj, long proj_stride,
-                                  int gate_column, T* __restrict__ out, int heads, int v, int n_tokens) {
+                                  int gate_column, T* __restrict__ out, int heads, int v, int n_tokens, int per_channel) {
+    // (per_channel: the gate of channel i of a head stands at column gate_column + head * v + i, not at gate_column + head)
     __shared__ float partial[4][64];
     const int t = blockIdx.x, head = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
@@ -129,14 +130,16 @@ __global__ void gate_heads_kernel(const T* __restrict__ y, const T* __restrict__
         for (int w = 0; w < waves; ++w) value += partial[w][lane];
     } else {                            // nothing to multiply: one workgroup gates the head's whole row
         float g = 1.f;
-        if (gate_column >= 0) g = 1.f / (1.f + expf(-(float)proj[(size_t)t * proj_stride + gate_column + head]));
-        for (int i = threadIdx.x; i < v; i += blockDim.x)
+        if (gate_column >= 0 && !per_channel) g = 1.f / (1.f + expf(-(float)proj[(size_t)t * proj_stride + gate_column + head]));
+        for (int i = threadIdx.x; i < v; i += blockDim.x) {
+            if (gate_column >= 0 && per_channel) g = 1.f / (1.f + expf(-(float)proj[(size_t)t * proj_stride + gate_column + (size_t)head * v + i]));
             out[((size_t)t * heads + head) * v + i] = (T)((float)y[((size_t)head * n_tokens + t) * v + i] * g);
+        }
         return;
     }
     if (j >= v) return;
     float g = 1.f;
-    if (gate_column >= 0) g = 1.f / (1.f + expf(-(float)proj[(size_t)t * proj_stride + gate_column + head]));
+    if (gate_column >= 0) g = 1.f / (1.f + expf(-(float)proj[(size_t)t * proj_stride + gate_column + (per_channel ? (size_t)head * v + j : (size_t)head)]));
     out[((size_t)t * heads + head) * v + j] = (T)(value * g);
 }
 
@@ -158,12 +161,13 @@ LSA_EXPORT int lsa_latent_prepare(int code, const void* proj, long proj_stride, 
 }
 
 LSA_EXPORT int lsa_gate_heads(int code, const void* y, const void* mixed, const void* up_values, int rank, int row_width, const void* proj,
-                              long proj_stride, int gate_column, void* out, int heads, int v, int n_tokens, hipStream_t stream) {
+                              long proj_stride, int gate_column, void* out, int heads, int v, int n_tokens, int per_channel,
+                              hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if ((y == nullptr) == (up_values == nullptr) || (up_values != nullptr && (mixed == nullptr || rank > row_width))) return -1;
     dim3 grid(n_tokens, heads, up_values ? (v + 63) / 64 : 1);
 #define LSA_LAUNCH(T) gate_heads_kernel<T><<<grid, up_values ? 256 : 64, 0, stream>>>((const T*)y, (const T*)mixed, (const T*)up_values, rank, row_width, \
-        (const T*)proj, proj_stride, gate_column, (T*)out, heads, v, n_tokens)
+        (const T*)proj, proj_stride, gate_column, (T*)out, heads, v, n_tokens, per_channel)
     if (code) LSA_LAUNCH(bf16_t); else LSA_LAUNCH(float);
 #undef LSA_LAUNCH
     LSA_LAUNCH_CHECK();

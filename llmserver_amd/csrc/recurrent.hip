@@ -1,6 +1,6 @@
 // Kernels of the mixers that carry a state of fixed size from token to token: the mix of a token's row with the row
-// before it, the linear recurrence S_t = diag(d_t) S_(t-1) + k_t v_t^T with its read-out, and the per-head norm and gate
-// behind it.  Decays, their exponentials and logarithms, the state, the sums and the norm are float32; projections
+// before it, the linear recurrence S_t = diag(d_t) S_(t-1) + k_t v_t^T with its read-out, the matrix memory with
+// exponential gates and a normaliser, and the per-head norm and gate behind them.  Decays, their exponentials and logarithms, the state, the sums and the norm are float32; projections
 // arrive in the activations' type and are widened where they are read; a result for a 16-bit consumer is rounded once.
 #include "common.hpp"
 
@@ -189,24 +189,210 @@ __global__ __launch_bounds__(512) void linear_recurrence_kernel(const T* __restr
         if (column_ok && channel0 + i < dim) mine[(size_t)i * value_dim] = S[i];
 }
 
-// grid (tokens, heads), one wavefront: out = x / rms(x) * w * silu(gate) over a head's value_dim numbers; x float32,
-// w = weight[head * weight_stride + j] (weight_stride 0: one weight shared by the heads), gate and out of type T.
+// grid (tokens, heads), one wavefront: out = x' / rms(x') * w * act(gate) over a head's value_dim numbers; x float32,
+// w = weight[head * weight_stride + j] (weight_stride 0: one weight shared by the heads), gate and out of type T;
+// act: gate * sigmoid(gate) (gate_kind 0) or sigmoid(gate) (1).  x' = x, or, with below [tokens][heads][2]:
+// x / (max(|below[0]|, below[1]) + floor), the read-out of a matrix memory under its normaliser.
 template <typename T>
 __global__ __launch_bounds__(64) void heads_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ weight, int weight_stride,
                                                              float eps, const T* __restrict__ gate, long gate_stride, T* __restrict__ out,
-                                                             int heads, int value_dim) {
+                                                             int heads, int value_dim, int gate_kind, const float* __restrict__ below,
+                                                             float floor) {
     const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const float* row = x + ((size_t)t * heads + head) * value_dim;
+    float under = 1.f;
+    if (below) {
+        const float* b = below + ((size_t)t * heads + head) * 2;
+        under = fmaxf(fabsf(b[0]), b[1]) + floor;
+    }
     float sq = 0.f;
-    for (int j = lane; j < value_dim; j += 64) sq += row[j] * row[j];
+    for (int j = lane; j < value_dim; j += 64) {
+        const float xv = below ? row[j] / under : row[j];
+        sq += xv * xv;
+    }
     const float inv = rsqrtf(wave_sum(sq) / (float)value_dim + eps);
     const T* g = gate + (size_t)t * gate_stride + (size_t)head * value_dim;
     const float* w = weight + (size_t)head * weight_stride;
     T* o = out + ((size_t)t * heads + head) * value_dim;
     for (int j = lane; j < value_dim; j += 64) {
         const float gv = (float)g[j];
-        o[j] = (T)(row[j] * inv * w[j] * (gv / (1.f + expf(-gv))));
+        const float sigmoid = 1.f / (1.f + expf(-gv));
+        const float xv = below ? row[j] / under : row[j];
+        o[j] = (T)(xv * inv * w[j] * (gate_kind ? sigmoid : gv * sigmoid));
     }
+}
+
+// ---- a matrix memory with exponential gates --------------------------------------------------------------------------
+// Per head and token: log input gate i = cap tanh(z_i / cap), log forget gate f = logsigmoid(cap tanh(z_f / cap)), a running
+// maximum m_t = max(f + m_(t-1), i) that starts at 0, and from them what the memory's update needs: keep = exp(f + m_(t-1) -
+// m_t), take = exp(i - m_t), and exp(-m_t) for the read-out's denominator.  grid (rows, heads), one wavefront: the row's
+// tokens in chunks of 64, a lane a token for the transcendental functions, one lane for the maximum's walk through the
+// chunk (two dependent instructions a token).  gates [T][2 heads] (inputs, then forgets), coef [T][heads][2] (keep, take),
+// below [T][heads][2] (its second number is written here), top[slot][head] the maximum between steps (0 at position 0).
+__global__ __launch_bounds__(64) void memory_gates_kernel(const float* __restrict__ gates, float cap, float* state, long state_stride,
+                                                          long top_offset, const int* __restrict__ slots, const int* __restrict__ row_start,
+                                                          const int* __restrict__ row_len, const int* __restrict__ row_ctx,
+                                                          float* __restrict__ coef, float* __restrict__ below, int heads) {
+    __shared__ float s_in[64], s_forget[64], s_top[65];
+    const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const int count = row_len[row];
+    if (count <= 0) return;
+    const int start = row_start[row], first_position = row_ctx[row] - count;
+    float* kept = state + (size_t)slots[row] * state_stride + top_offset + head;
+    float top = first_position > 0 ? *kept : 0.f;                      // (the same number in every lane)
+    const float inv_cap = 1.f / cap;
+    for (int t0 = 0; t0 < count; t0 += 64) {
+        const int n = min(64, count - t0);
+        const size_t token = (size_t)(start + t0 + lane);
+        float log_in = 0.f, log_forget = 0.f;
+        if (lane < n) {
+            log_in = cap * tanhf(gates[token * 2 * heads + head] * inv_cap);
+            const float z = cap * tanhf(gates[token * 2 * heads + heads + head] * inv_cap);
+            log_forget = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+        }
+        __syncthreads();                                               // the chunk before has been read
+        s_in[lane] = log_in;
+        s_forget[lane] = log_forget;
+        __syncthreads();
+        if (lane == 0) {
+            float m = top;
+            s_top[0] = m;
+            for (int t = 0; t < n; ++t) {
+                m = fmaxf(s_forget[t] + m, s_in[t]);
+                s_top[t + 1] = m;
+            }
+        }
+        __syncthreads();
+        if (lane < n) {
+            const float before = s_top[lane], now = s_top[lane + 1];
+            coef[(token * heads + head) * 2] = expf((log_forget + before) - now);
+            coef[(token * heads + head) * 2 + 1] = expf(log_in - now);
+            below[(token * heads + head) * 2 + 1] = expf(-now);
+        }
+        top = s_top[n];
+    }
+    if (lane == 0) *kept = top;
+}
+
+// One token of one wavefront's DK channels of a matrix memory: S = keep S + k value (value: the token's value column times its
+// take), and the channels' part of the read-out S^T q; the channels come from LDS as in recurrence_token.
+template <int DK>
+__device__ __forceinline__ float memory_token(float (&S)[DK], const float* q_row, const float* k_row, float keep, float value) {
+    const float4* tq = reinterpret_cast<const float4*>(q_row);
+    const float4* tk = reinterpret_cast<const float4*>(k_row);
+    float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i4 = 0; i4 < DK / 4; ++i4) {
+        const float4 q4 = tq[i4], k4 = tk[i4];
+        const float qs[4] = {q4.x, q4.y, q4.z, q4.w}, ks[4] = {k4.x, k4.y, k4.z, k4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int i = 4 * i4 + e;
+            S[i] = __builtin_fmaf(keep, S[i], ks[e] * value);
+            o4[e] = __builtin_fmaf(S[i], qs[e], o4[e]);
+        }
+    }
+    return (o4[0] + o4[1]) + (o4[2] + o4[3]);
+}
+
+// The memory itself, laid out as linear_recurrence_kernel: grid (rows, heads, blocks of 64 columns), lane = column,
+// wavefront w owns key channels [w * DK, (w + 1) * DK) and keeps its piece of the state in registers over the row's tokens.
+// The columns are the head's value_dim value columns and, behind them, one more whose "value" is 1: its piece of the state
+// is the normaliser n, which obeys the same recurrence with k in place of k v^T, and its read-out is n . q.  So
+// out [T][heads * value_dim] gets the numerators S^T q and below [T][heads][2] (first number) gets n . q; the division is
+// left to the kernel that normalises the heads.  state[slot]: the matrices [heads][dim][value_dim], then the normalisers
+// [heads][dim].  Every sum is formed in the same order however the sequence was cut into steps.
+template <typename T, int DK>
+__global__ __launch_bounds__(512) void matrix_memory_kernel(const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
+                                         const T* __restrict__ v, long v_stride, const float* __restrict__ coef, float q_scale,
+                                         float* state, long state_stride, const int* __restrict__ slots,
+                                         const int* __restrict__ row_start, const int* __restrict__ row_len, const int* __restrict__ row_ctx,
+                                         float* __restrict__ out, float* __restrict__ below, int heads, int dim, int value_dim) {
+    extern __shared__ __align__(16) float lds[];
+    const int row = blockIdx.x, head = blockIdx.y, column0 = blockIdx.z * 64;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int count = row_len[row];
+    if (count <= 0) return;                              // (the whole workgroup: nobody waits at a barrier below)
+    const int start = row_start[row], first_position = row_ctx[row] - count;
+    const int padded = waves * DK;                       // channels as the wavefronts share them; those behind dim are zeros
+    float* s_q = lds;                                    // [CHUNK][padded]
+    float* s_k = s_q + CHUNK * padded;
+    float* s_v = s_k + CHUNK * padded;                   // [CHUNK][64], each value times its token's take
+    float* s_keep = s_v + CHUNK * 64;                    // [CHUNK]
+    float* s_o = s_keep + CHUNK;                         // [waves][CHUNK][64]
+    const int column = column0 + lane;
+    const bool is_value = column < value_dim, is_normaliser = column == value_dim;
+    const int channel0 = wave * DK;
+    float* slot = state + (size_t)slots[row] * state_stride;
+    // a channel's number of this column: in the matrix, or in the normaliser behind the matrices
+    float* mine = is_value ? slot + ((size_t)head * dim + channel0) * value_dim + column
+                           : slot + (size_t)heads * dim * value_dim + (size_t)head * dim + channel0;
+    const size_t channel_stride = is_value ? (size_t)value_dim : 1;
+    float S[DK];
+#pragma unroll
+    for (int i = 0; i < DK; ++i) {
+        const bool ok = (is_value || is_normaliser) && channel0 + i < dim;
+        S[i] = (ok && first_position > 0) ? mine[(size_t)i * channel_stride] : 0.f;
+    }
+    const size_t key_column = (size_t)head * dim;
+    for (int t0 = 0; t0 < count; t0 += CHUNK) {
+        const int n = min(CHUNK, count - t0);
+        __syncthreads();                                 // the chunk before has been read out of LDS
+        constexpr int PER = CHUNK * DK / 64;
+        float raw_q[PER], raw_k[PER];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            const int t = i / padded, c = i - t * padded;
+            raw_q[j] = 0.f; raw_k[j] = 0.f;
+            if (t < n && c < dim) {
+                const size_t token = (size_t)(start + t0 + t);
+                raw_q[j] = (float)q[token * q_stride + key_column + c];
+                raw_k[j] = (float)k[token * k_stride + key_column + c];
+            }
+        }
+        for (int i = threadIdx.x; i < n * 64; i += blockDim.x) {
+            const int t = i >> 6, c = column0 + (i & 63);
+            const size_t token = (size_t)(start + t0 + t);
+            const float take = coef[(token * heads + head) * 2 + 1];
+            const float value = c < value_dim ? (float)v[token * v_stride + (size_t)head * value_dim + c] : (c == value_dim ? 1.f : 0.f);
+            s_v[i] = take * value;
+        }
+        if (threadIdx.x < n) s_keep[threadIdx.x] = coef[((size_t)(start + t0 + threadIdx.x) * heads + head) * 2];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            if (i / padded >= n) continue;
+            s_q[i] = raw_q[j] * q_scale;
+            s_k[i] = raw_k[j];
+        }
+        __syncthreads();
+        if (DK <= 16 && n == CHUNK) {
+            float kept[CHUNK];
+#pragma unroll
+            for (int t = 0; t < CHUNK; ++t)
+                kept[t] = memory_token<DK>(S, s_q + t * padded + channel0, s_k + t * padded + channel0, s_keep[t], s_v[t * 64 + lane]);
+#pragma unroll
+            for (int t = 0; t < CHUNK; ++t) s_o[(wave * CHUNK + t) * 64 + lane] = kept[t];
+        } else {
+            for (int t = 0; t < n; ++t)
+                s_o[(wave * CHUNK + t) * 64 + lane] = memory_token<DK>(S, s_q + t * padded + channel0, s_k + t * padded + channel0,
+                                                                       s_keep[t], s_v[t * 64 + lane]);
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < n * 64; i += blockDim.x) {
+            const int t = i >> 6, c = column0 + (i & 63);
+            if (c > value_dim) continue;
+            float total = 0.f;
+            for (int w = 0; w < waves; ++w) total += s_o[(w * CHUNK + t) * 64 + (i & 63)];
+            const size_t token = (size_t)(start + t0 + t);
+            if (c < value_dim) out[token * heads * value_dim + (size_t)head * value_dim + c] = total;
+            else below[(token * heads + head) * 2] = total;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < DK; ++i)
+        if ((is_value || is_normaliser) && channel0 + i < dim) mine[(size_t)i * channel_stride] = S[i];
 }
 
 template <typename T>
@@ -273,6 +459,14 @@ LSA_EXPORT int lsa_recurrent_prepare() {
     LSA_ALLOW_ALL(bf16_t);
 #undef LSA_ALLOW_ALL
 #undef LSA_ALLOW
+#define LSA_ALLOW(T, DK) do { \
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&matrix_memory_kernel<T, DK>), \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, MOST_LDS); \
+        if (e != hipSuccess && first == hipSuccess) first = e; \
+    } while (0)
+    LSA_ALLOW(float, 8); LSA_ALLOW(float, 16); LSA_ALLOW(float, 32); LSA_ALLOW(float, 64);
+    LSA_ALLOW(bf16_t, 8); LSA_ALLOW(bf16_t, 16); LSA_ALLOW(bf16_t, 32); LSA_ALLOW(bf16_t, 64);
+#undef LSA_ALLOW
     (void)hipGetLastError();
     return (int)first;
 }
@@ -300,12 +494,40 @@ LSA_EXPORT int lsa_linear_recurrence(int code, const void* q, long q_stride, con
 }
 
 LSA_EXPORT int lsa_heads_norm_gate(int code, const float* x, const float* weight, int weight_per_channel, float eps, const void* gate,
-                                   long gate_stride, void* out, int n_tokens, int heads, int value_dim, hipStream_t stream) {
+                                   long gate_stride, void* out, int n_tokens, int heads, int value_dim, int gate_kind, const float* below,
+                                   float floor, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (gate_kind != 0 && gate_kind != 1) return -1;
     dim3 grid(n_tokens, heads);
     const int weight_stride = weight_per_channel ? value_dim : 0;
-    if (code) heads_norm_gate_kernel<bf16_t><<<grid, 64, 0, stream>>>(x, weight, weight_stride, eps, (const bf16_t*)gate, gate_stride, (bf16_t*)out, heads, value_dim);
-    else heads_norm_gate_kernel<float><<<grid, 64, 0, stream>>>(x, weight, weight_stride, eps, (const float*)gate, gate_stride, (float*)out, heads, value_dim);
+    if (code) heads_norm_gate_kernel<bf16_t><<<grid, 64, 0, stream>>>(x, weight, weight_stride, eps, (const bf16_t*)gate, gate_stride, (bf16_t*)out, heads, value_dim, gate_kind, below, floor);
+    else heads_norm_gate_kernel<float><<<grid, 64, 0, stream>>>(x, weight, weight_stride, eps, (const float*)gate, gate_stride, (float*)out, heads, value_dim, gate_kind, below, floor);
+    LSA_LAUNCH_CHECK();
+}
+
+// state[slot]: the matrices [heads][dim][value_dim], the normalisers [heads][dim], the maxima [heads].
+LSA_EXPORT int lsa_matrix_memory(int code, const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
+                                 const float* gates, float cap, float q_scale, float* state, long state_stride, const int* slots,
+                                 const int* row_start, const int* row_len, const int* row_ctx, float* coef, float* out, float* below,
+                                 int rows, int heads, int dim, int value_dim, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dim < 1 || dim > MOST_DIM || value_dim < 1 || heads < 1 || !(cap > 0.f) || state == nullptr || coef == nullptr || below == nullptr) return -1;
+    if (state_stride < (long)heads * dim * value_dim + (long)heads * dim + heads) return -1;
+    int dk, waves;
+    recurrence_lds(dim, dk, waves);
+    const size_t lds = sizeof(float) * ((size_t)2 * CHUNK * waves * dk + (size_t)CHUNK * 64 + CHUNK + (size_t)waves * CHUNK * 64);
+    if (lds > (size_t)MOST_LDS) return -1;
+    memory_gates_kernel<<<dim3(rows, heads), 64, 0, stream>>>(gates, cap, state, state_stride, (long)heads * dim * value_dim + (long)heads * dim,
+                                                              slots, row_start, row_len, row_ctx, coef, below, heads);
+    dim3 grid(rows, heads, (value_dim + 1 + 63) / 64);
+#define LSA_LAUNCH(T, DK) \
+        matrix_memory_kernel<T, DK><<<grid, waves * 64, lds, stream>>>((const T*)q, q_stride, (const T*)k, k_stride, (const T*)v, v_stride, \
+            coef, q_scale, state, state_stride, slots, row_start, row_len, row_ctx, out, below, heads, dim, value_dim)
+#define LSA_BY_DK(T) do { if (dk == 8) LSA_LAUNCH(T, 8); else if (dk == 16) LSA_LAUNCH(T, 16); else if (dk == 32) LSA_LAUNCH(T, 32); \
+                          else LSA_LAUNCH(T, 64); } while (0)
+    if (code) LSA_BY_DK(bf16_t); else LSA_BY_DK(float);
+#undef LSA_BY_DK
+#undef LSA_LAUNCH
     LSA_LAUNCH_CHECK();
 }
 

@@ -280,7 +280,7 @@ __global__ __launch_bounds__(64) void qkv_prepare_kernel(const T* __restrict__ q
                                                          const int* __restrict__ positions, const float* __restrict__ q_weight,
                                                          const float* __restrict__ k_weight, float eps, const float* __restrict__ cos_sin,
                                                          int pairs, int page_size, int n_q, int n_kv, int dim, int value_dim, int D,
-                                                         T* __restrict__ out_q, int write_cache) {
+                                                         T* __restrict__ out_q, int write_cache, int halves) {
     const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const bool is_query = head < n_q;
     if (!is_query && !write_cache) return;
@@ -299,8 +299,13 @@ __global__ __launch_bounds__(64) void qkv_prepare_kernel(const T* __restrict__ q
     auto prepared = [&](int e) -> float {
         if (e >= dim) return 0.f;
         auto normed = [&](int i) { return weight ? (float)src[i] * inv * weight[i] : (float)src[i]; };
+        if (!cs || e >= 2 * pairs) return normed(e);
+        if (halves) {                                      // dimension i turns with dimension i + pairs
+            const int pair = e < pairs ? e : e - pairs;
+            const float u = normed(pair), w = normed(pair + pairs), c = cs[pair], s = cs[pairs + pair];
+            return e < pairs ? u * c - w * s : w * c + u * s;
+        }
         const int pair = e >> 1;
-        if (!cs || pair >= pairs) return normed(e);
         const float u = normed(2 * pair), w = normed(2 * pair + 1), c = cs[pair], s = cs[pairs + pair];
         return (e & 1) ? w * c + u * s : u * c - w * s;
     };
@@ -325,12 +330,12 @@ __global__ __launch_bounds__(64) void qkv_prepare_kernel(const T* __restrict__ q
 LSA_EXPORT int lsa_qkv_prepare(int dtype, const void* qkv, long stride, void* keys, void* values, const int* table, int table_stride,
                                const int* token_row, const int* positions, const float* q_weight, const float* k_weight, float eps,
                                const float* cos_sin, int pairs, int page_size, int n_q, int n_kv, int dim, int value_dim, int D,
-                               void* out_q, int write_cache, int n_tokens, hipStream_t stream) {
+                               void* out_q, int write_cache, int n_tokens, int halves, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (dim > D || value_dim > D || 2 * pairs > dim || page_size <= 0 || (q_weight == nullptr) != (k_weight == nullptr)) return -1;
     dim3 grid(n_tokens, n_q + n_kv);
 #define LSA_LAUNCH(T) qkv_prepare_kernel<T><<<grid, 64, 0, stream>>>((const T*)qkv, stride, (T*)keys, (T*)values, table, table_stride, token_row, \
-        positions, q_weight, k_weight, eps, cos_sin, pairs, page_size, n_q, n_kv, dim, value_dim, D, (T*)out_q, write_cache)
+        positions, q_weight, k_weight, eps, cos_sin, pairs, page_size, n_q, n_kv, dim, value_dim, D, (T*)out_q, write_cache, halves)
     if (dtype) LSA_LAUNCH(bf16_t); else LSA_LAUNCH(float);
 #undef LSA_LAUNCH
     LSA_LAUNCH_CHECK();

@@ -1,7 +1,8 @@
 // Row-wise kernels around a residual stream that is kept in float32 whatever the type of the activations:
 // embedding lookup with the norm behind it, a norm of chosen rows, a short causal convolution over time with a
-// per-request state, and the update behind a sublayer (norm of the sublayer's result, per-channel scale, sum, and
-// the weighted sum over the results of the layers so far).  One workgroup per token row; sums of squares, rsqrt and
+// per-request state, the update behind a sublayer (norm of the sublayer's result, per-channel scale, sum, and
+// the weighted sum over the results of the layers so far), and several such streams side by side that sublayers read
+// as a weighted sum and update all at once.  One workgroup per token row; sums of squares, rsqrt and
 // every sum are 32-bit; a result for a 16-bit consumer is rounded once when it is stored.
 #include "common.hpp"
 
@@ -180,15 +181,104 @@ __global__ __launch_bounds__(256) void scaled_norm_add_kernel(const float* __res
     }
 }
 
-// out[t] = table[ids[t]] widened to float32 (an id outside the table gives a zero row).
+// out[c][t] = table[ids[t]] * scale, widened to float32, for each of `copies` equal copies (several residual streams start
+// alike); an id outside the table gives a zero row.
 template <typename T>
 __global__ __launch_bounds__(256) void embedding_wide_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                                                             float* __restrict__ out, int width, int vocab) {
+                                                             float* __restrict__ out, int width, int vocab, float scale, int copies,
+                                                             size_t copy_stride) {
     const int id = ids[blockIdx.x];
     const bool ok = id >= 0 && id < vocab;
     const T* row = table + (size_t)(ok ? id : 0) * width;
     float* o = out + (size_t)blockIdx.x * width;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = ok ? (float)row[i] : 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float value = ok ? (float)row[i] * scale : 0.f;
+        for (int c = 0; c < copies; ++c) o[(size_t)c * copy_stride + i] = value;
+    }
+}
+
+// ---- several residual streams x [S][T][W], float32 ------------------------------------------------------------------------
+constexpr int MOST_STREAMS = 8;
+constexpr int STREAM_CACHE = 8;           // elements of a row a thread keeps between the two passes (rows of up to 2,048 are read once)
+
+// out[i] = rmsnorm(sum_s read[s] * x[s][rows[i]]) * weight (rows == nullptr: every row).
+template <typename O>
+__global__ __launch_bounds__(256) void streams_read_kernel(const float* __restrict__ x, size_t stream_stride, int streams,
+                                                           const float* __restrict__ read, const int* __restrict__ rows,
+                                                           const float* __restrict__ weight, float eps, O* __restrict__ out, int width) {
+    __shared__ float scratch[16];
+    const float* row = x + (size_t)(rows ? rows[blockIdx.x] : blockIdx.x) * width;
+    float r[MOST_STREAMS];
+    for (int s = 0; s < MOST_STREAMS; ++s) r[s] = s < streams ? read[s] : 0.f;
+    auto summed = [&](int i) {
+        float u = 0.f;
+        for (int s = 0; s < streams; ++s) u += r[s] * row[(size_t)s * stream_stride + i];
+        return u;
+    };
+    float kept[STREAM_CACHE];
+    float sq = 0.f;
+    int k = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++k) {
+        const float u = summed(i);
+        if (k < STREAM_CACHE) kept[k] = u;
+        sq += u * u;
+    }
+    const float inv = rsqrtf(block_sum(sq, scratch) / (float)width + eps);
+    O* o = out + (size_t)blockIdx.x * width;
+    k = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++k) o[i] = (O)((k < STREAM_CACHE ? kept[k] : summed(i)) * inv * weight[i]);
+}
+
+// All streams at once from the old ones, where they lie: x[t] <- sum_s mix[s][t] * x[s] + write[t] * y, and, where next_read
+// is given, normed = rmsnorm(sum_t next_read[t] * x[t]) * next_weight: what the next sublayer reads, in the same pass (the
+// row of sums stays in registers between the two passes; wider rows are formed again from the streams just written, by the
+// thread that wrote them).  One workgroup a token row.
+template <typename Y, typename R>
+__global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__ x, size_t stream_stride, int streams, const Y* __restrict__ y,
+                                                             const float* __restrict__ mix, const float* __restrict__ write,
+                                                             const float* __restrict__ next_read, const float* __restrict__ next_weight,
+                                                             float next_eps, R* __restrict__ normed, int width) {
+    __shared__ float scratch[16];
+    __shared__ float s_mix[MOST_STREAMS * MOST_STREAMS], s_write[MOST_STREAMS], s_read[MOST_STREAMS];
+    if (threadIdx.x < streams * streams) s_mix[threadIdx.x] = mix[threadIdx.x];
+    if (threadIdx.x < streams) {
+        s_write[threadIdx.x] = write[threadIdx.x];
+        s_read[threadIdx.x] = next_read ? next_read[threadIdx.x] : 0.f;
+    }
+    __syncthreads();
+    float* row = x + (size_t)blockIdx.x * width;
+    const Y* yr = y + (size_t)blockIdx.x * width;
+    float kept[STREAM_CACHE];
+    float sq = 0.f;
+    int k = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++k) {
+        float old[MOST_STREAMS];
+        for (int s = 0; s < streams; ++s) old[s] = row[(size_t)s * stream_stride + i];
+        const float update = (float)yr[i];
+        float u = 0.f;
+        for (int t = 0; t < streams; ++t) {
+            float fresh = 0.f;
+            for (int s = 0; s < streams; ++s) fresh += s_mix[s * streams + t] * old[s];
+            fresh += s_write[t] * update;
+            row[(size_t)t * stream_stride + i] = fresh;
+            u += s_read[t] * fresh;
+        }
+        if (k < STREAM_CACHE) kept[k] = u;
+        sq += u * u;
+    }
+    if (!next_read) return;                              // (the whole workgroup)
+    const float inv = rsqrtf(block_sum(sq, scratch) / (float)width + next_eps);
+    R* o = normed + (size_t)blockIdx.x * width;
+    k = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++k) {
+        float u;
+        if (k < STREAM_CACHE) u = kept[k];
+        else {
+            u = 0.f;
+            for (int t = 0; t < streams; ++t) u += s_read[t] * row[(size_t)t * stream_stride + i];
+        }
+        o[i] = (R)(u * inv * next_weight[i]);
+    }
 }
 
 // s = x + u * rsqrt(mean(u^2) + eps) * weight with u = y, or a * y + b * y2 where y2 is given; out = s; and where
@@ -266,10 +356,41 @@ __global__ __launch_bounds__(256) void norm_add_norm_kernel(const float* __restr
 }
 
 LSA_EXPORT int lsa_embedding_wide(int table_code, const void* table, const int* ids, float* out, int n, int width, int vocab,
-                                  hipStream_t stream) {
+                                  float scale, int copies, hipStream_t stream) {
     if (n <= 0) return 0;
-    if (table_code) embedding_wide_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)table, ids, out, width, vocab);
-    else embedding_wide_kernel<float><<<n, 256, 0, stream>>>((const float*)table, ids, out, width, vocab);
+    if (copies < 1) return -1;
+    const size_t copy_stride = (size_t)n * width;
+    if (table_code) embedding_wide_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)table, ids, out, width, vocab, scale, copies, copy_stride);
+    else embedding_wide_kernel<float><<<n, 256, 0, stream>>>((const float*)table, ids, out, width, vocab, scale, copies, copy_stride);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_most_streams() { return MOST_STREAMS; }
+
+// x [streams][n_tokens][width]; out [n_out][width].
+LSA_EXPORT int lsa_streams_read(const float* x, int streams, int n_tokens, const float* read, const int* rows, const float* weight, float eps,
+                                void* out, int out_code, int n_out, int width, hipStream_t stream) {
+    if (n_out <= 0) return 0;
+    if (streams < 1 || streams > MOST_STREAMS) return -1;
+    const size_t stream_stride = (size_t)n_tokens * width;
+    if (out_code) streams_read_kernel<bf16_t><<<n_out, 256, 0, stream>>>(x, stream_stride, streams, read, rows, weight, eps, (bf16_t*)out, width);
+    else streams_read_kernel<float><<<n_out, 256, 0, stream>>>(x, stream_stride, streams, read, rows, weight, eps, (float*)out, width);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_streams_update(float* x, int streams, int n_tokens, const void* y, int y_code, const float* mix, const float* write,
+                                  const float* next_read, const float* next_weight, float next_eps, void* normed, int normed_code, int width,
+                                  hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (streams < 1 || streams > MOST_STREAMS || (next_read != nullptr && (normed == nullptr || next_weight == nullptr))) return -1;
+    const size_t stream_stride = (size_t)n_tokens * width;
+#define LSA_LAUNCH(Y, R) streams_update_kernel<Y, R><<<n_tokens, 256, 0, stream>>>(x, stream_stride, streams, (const Y*)y, mix, write, next_read, \
+                                                                                  next_weight, next_eps, (R*)normed, width)
+    if (y_code && normed_code) LSA_LAUNCH(bf16_t, bf16_t);
+    else if (y_code) LSA_LAUNCH(bf16_t, float);
+    else if (normed_code) LSA_LAUNCH(float, bf16_t);
+    else LSA_LAUNCH(float, float);
+#undef LSA_LAUNCH
     LSA_LAUNCH_CHECK();
 }
 

@@ -25,17 +25,23 @@ _SIGNATURES = {
     "lsa_sample_static_error": [c_int],
     "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P, _P, _P, _P, c_int,
                             c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P, c_float, _P],
-    "lsa_embedding_wide": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_embedding_wide": [c_int, _P, _P, _P, c_int, c_int, c_int, c_float, c_int, _P],
+    "lsa_most_streams": [],
+    "lsa_streams_read": [_P, c_int, c_int, _P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
+    "lsa_streams_update": [_P, c_int, c_int, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, _P],
+    "lsa_activation": [c_int, _P, c_long, c_int, _P],
+    "lsa_matrix_memory": [c_int, _P, c_long, _P, c_long, _P, c_long, _P, c_float, c_float, _P, c_long, _P, _P, _P, _P, _P, _P, _P,
+                          c_int, c_int, c_int, c_int, _P],
     "lsa_norm_add_norm": [_P, _P, _P, c_int, c_float, c_float, _P, c_float, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_qkv_prepare": [c_int, _P, c_long, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                        _P, c_int, c_int, _P],
+                        _P, c_int, c_int, c_int, _P],
     "lsa_token_shift": [c_int, _P, _P, c_int, _P, c_long, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
     "lsa_token_shift_keep": [c_int, _P, _P, c_long, _P, _P, _P, c_int, c_int, _P],
     "lsa_linear_recurrence_most_dim": [],
     "lsa_recurrent_prepare": [],
     "lsa_linear_recurrence": [c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, c_float, _P, c_float, _P, c_long, _P, _P, _P, _P, _P,
                               c_int, c_int, c_int, c_int, _P],
-    "lsa_heads_norm_gate": [c_int, _P, _P, c_int, c_float, _P, c_long, _P, c_int, c_int, c_int, _P],
+    "lsa_heads_norm_gate": [c_int, _P, _P, c_int, c_float, _P, c_long, _P, c_int, c_int, c_int, c_int, _P, c_float, _P],
     "lsa_tanh": [c_int, _P, c_long, _P],
     "lsa_scaled_sum": [c_int, _P, c_float, _P, c_float, _P, c_long, _P],
     "lsa_embedding_norm": [c_int, _P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
@@ -45,7 +51,7 @@ _SIGNATURES = {
     "lsa_scaled_norm_add": [_P, _P, c_int, _P, _P, c_float, _P, _P, c_int, _P, c_long, c_int, _P, c_int, c_int, _P],
     "lsa_latent_prepare": [c_int, _P, c_long, _P, _P, _P, c_float, _P, c_int, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int,
                            c_int, c_int, c_int, c_int, _P],
-    "lsa_gate_heads": [c_int, _P, _P, _P, c_int, c_int, _P, c_long, c_int, _P, c_int, c_int, c_int, _P],
+    "lsa_gate_heads": [c_int, _P, _P, _P, c_int, c_int, _P, c_long, c_int, _P, c_int, c_int, c_int, c_int, _P],
     "lsa_route_logits": [_P, _P, _P, c_int, c_int, c_int, _P],
     "lsa_route_top": [_P, c_int, c_int, _P, _P, c_int, c_int, c_int, c_int, _P],
     "lsa_experts_gate_up": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P],

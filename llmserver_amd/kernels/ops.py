@@ -798,15 +798,57 @@ class HipOps(KernelNamespace):
         _launched(self._part_library("stream").lsa_embedding_norm(_code(table), _ptr(table), _ptr(token_ids), _ptr(weight), float(eps),
                                                                   _ptr(out), n, width, table.shape[0], _stream()), "embedding_norm")
 
-    def embedding_wide(self, table, token_ids, out):
-        n, width = out.shape
+    def embedding_wide(self, table, token_ids, out, scale=1.0):
+        copies = out.shape[0] if out.dim() == 3 else 1          # several residual streams start as equal copies of the rows
+        n, width = out.shape[-2:]
         _check(table, "table")
         _check(token_ids, "token_ids", torch.int32, (n,))
         _check(out, "out", torch.float32)
         if table.shape[1] != width:
             raise ValueError(f"embedding: table width {table.shape[1]} != out width {width}")
         _launched(self._part_library("stream").lsa_embedding_wide(_code(table), _ptr(table), _ptr(token_ids), _ptr(out), n, width,
-                                                                  table.shape[0], _stream()), "embedding_wide")
+                                                                  table.shape[0], float(scale), copies, _stream()), "embedding_wide")
+
+    def _check_streams(self, streams):
+        _check(streams, "streams", torch.float32)
+        most = self._part_library("stream").lsa_most_streams()
+        if streams.dim() != 3 or not 1 <= streams.shape[0] <= most:
+            raise ValueError(f"residual streams come as [streams, T, W] with up to {most} streams, got {tuple(streams.shape)}")
+        return streams.shape
+
+    def streams_read(self, streams, read, weight, eps, out, rows=None):
+        count, n, width = self._check_streams(streams)
+        n_out = n if rows is None else rows.shape[0]
+        _check(read, "read", torch.float32, (count,))
+        _check(weight, "weight", torch.float32, (width,))
+        _check(out, "out", None, (n_out, width))
+        if rows is not None:
+            _check(rows, "rows", torch.int32, (n_out,))
+        _launched(self._part_library("stream").lsa_streams_read(_ptr(streams), count, n, _ptr(read), _ptr(rows), _ptr(weight), float(eps),
+                                                                _ptr(out), _code(out), n_out, width, _stream()), "streams_read")
+
+    def streams_update(self, streams, y, mix, write, next_read=None, next_weight=None, next_eps=0.0, normed=None):
+        count, n, width = self._check_streams(streams)
+        _check(y, "y", None, (n, width))
+        _check(mix, "mix", torch.float32, (count, count))
+        _check(write, "write", torch.float32, (count,))
+        if next_read is not None:
+            _check(next_read, "next_read", torch.float32, (count,))
+            _check(next_weight, "next_weight", torch.float32, (width,))
+            _check(normed, "normed", None, (n, width))
+        _launched(self._part_library("stream").lsa_streams_update(
+            _ptr(streams), count, n, _ptr(y), _code(y), _ptr(mix), _ptr(write), _ptr(next_read),
+            _ptr(next_weight) if next_read is not None else None, float(next_eps), _ptr(normed) if next_read is not None else None,
+            _code(normed) if next_read is not None else 0, width, _stream()), "streams_update")
+
+    PLAIN_ACTIVATIONS = ("silu", "gelu_tanh", "relu2")     # what the ungated activation kernel computes (its codes)
+
+    def activation_(self, x, activation):
+        if activation not in self.PLAIN_ACTIVATIONS:
+            raise ValueError(f"the activation kernel computes {', '.join(self.PLAIN_ACTIVATIONS)}; {activation!r} is not built")
+        _check(x, "x")
+        _launched(self._elementwise.lsa_activation(_code(x), _ptr(x), x.numel(), self.PLAIN_ACTIVATIONS.index(activation), _stream()),
+                  "activation")
 
     def norm_add_norm(self, x, y, weight, eps, out, next_weight=None, next_eps=0.0, normed=None, y2=None, scales=None):
         n, width = x.shape
@@ -928,7 +970,7 @@ class HipOps(KernelNamespace):
             _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(token_row), _ptr(positions), page_size, _ptr(out_q), n_heads, dim,
             rot_dim, rank, row_width, 1 if write_cache else 0, n, _stream()), "latent_prepare")
 
-    def gate_heads(self, y, proj, gate_column, out, mixed=None, up_values=None):
+    def gate_heads(self, y, proj, gate_column, out, mixed=None, up_values=None, per_channel=False):
         _check(proj, "proj", out.dtype)
         _check(out, "out")
         n = out.shape[0]
@@ -945,10 +987,12 @@ class HipOps(KernelNamespace):
             row_width = mixed.shape[1] // heads
             if mixed.shape != (n, heads * row_width) or rank > row_width:
                 raise ValueError(f"mixed {tuple(mixed.shape)} does not hold {heads} rows of at least {rank} a token")
-        if tuple(out.shape) != (n, heads * v) or proj.shape[0] != n or gate_column + heads > proj.shape[1]:
-            raise ValueError(f"gates of {heads} heads from column {gate_column} of proj {tuple(proj.shape)} for an output of {tuple(out.shape)}")
+        gates = heads * v if per_channel else heads
+        if tuple(out.shape) != (n, heads * v) or proj.shape[0] != n or gate_column + gates > proj.shape[1]:
+            raise ValueError(f"{gates} gates of {heads} heads from column {gate_column} of proj {tuple(proj.shape)} for an output of {tuple(out.shape)}")
         _launched(self._part_library("latent").lsa_gate_heads(_code(out), _ptr(y), _ptr(mixed), _ptr(up_values), rank, row_width, _ptr(proj),
-                                                              proj.shape[1], int(gate_column), _ptr(out), heads, v, n, _stream()), "gate_heads")
+                                                              proj.shape[1], int(gate_column), _ptr(out), heads, v, n, 1 if per_channel else 0,
+                                                              _stream()), "gate_heads")
 
     def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None):
         """The logits are a float32 product of the library (no reduced-precision mode), the choice and the weights a kernel."""
@@ -1032,8 +1076,10 @@ class HipOps(KernelNamespace):
 
     # -- general preparation of queries, keys and values; mixers with a recurrent state -----------------------------
     def qkv_prepare(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
-                    n_q, n_kv, dim, value_dim, out_q, write_cache=True):
+                    n_q, n_kv, dim, value_dim, out_q, write_cache=True, pairing="neighbours"):
         n = qkv.shape[0]
+        if pairing not in ("neighbours", "halves"):
+            raise ValueError(f"dimensions turn in neighbouring pairs or in halves, not {pairing!r}")
         _check(qkv, "qkv", None, (n, (n_q + n_kv) * dim + n_kv * value_dim))
         pages, row = keys.shape[0], keys.shape[-1]
         _check(keys, "keys", qkv.dtype, (pages, n_kv, page_size, row))
@@ -1058,7 +1104,7 @@ class HipOps(KernelNamespace):
         _launched(self._rope_kv.lsa_qkv_prepare(
             _code(qkv), _ptr(qkv), qkv.shape[1], _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(token_row), _ptr(positions),
             _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin), pairs, page_size, n_q, n_kv, dim, value_dim, row, _ptr(out_q),
-            1 if write_cache else 0, n, _stream()), "qkv_prepare")
+            1 if write_cache else 0, n, 1 if pairing == "halves" else 0, _stream()), "qkv_prepare")
 
     @staticmethod
     def _state_rows(state, offset, needed, name):
@@ -1138,8 +1184,36 @@ class HipOps(KernelNamespace):
             self.DECAY_MODES.index(decay_mode), float(tau), _ptr(bonus), float(q_scale), pointer, stride, _ptr(state_slots), _ptr(row_start),
             _ptr(row_len), _ptr(row_ctx), _ptr(out), rows, heads, dim, value_dim, _stream()), "linear_recurrence")
 
-    def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim):
+    GATE_ACTIVATIONS = ("silu", "sigmoid")
+
+    def matrix_memory(self, q, k, v, gates, cap, q_scale, state, state_slots, row_start, row_len, row_ctx, out, below, coefficients,
+                      heads, dim, value_dim):
+        n = out.shape[0]
+        rows = row_len.shape[0]
+        lib = self._part_library("recurrent")
+        if dim > lib.lsa_linear_recurrence_most_dim():
+            raise ValueError(f"the memory kernel takes heads of up to {lib.lsa_linear_recurrence_most_dim()} key channels, got {dim}")
+        for name, tensor, columns in (("q", q, heads * dim), ("k", k, heads * dim), ("v", v, heads * value_dim)):
+            if not tensor.is_cuda or tensor.dtype != q.dtype or tuple(tensor.shape) != (n, columns) or (n > 1 and tensor.stride(1) != 1):
+                raise ValueError(f"{name} must be a view [{n}, {columns}] of {q.dtype} on the GPU with unit stride along a row")
+        _check(gates, "gates", torch.float32, (n, 2 * heads))
+        _check(out, "out", torch.float32, (n, heads * value_dim))
+        _check(below, "below", torch.float32, (n, heads, 2))
+        for name, tensor in (("state_slots", state_slots), ("row_start", row_start), ("row_len", row_len), ("row_ctx", row_ctx)):
+            _check(tensor, name, torch.int32, (rows,))
+        pointer, stride = self._state_rows(state, 0, heads * dim * value_dim + heads * dim + heads, "state")
+        _check(coefficients, "coefficients", torch.float32, (n, heads, 2))
+        _launched(lib.lsa_matrix_memory(
+            _code(q), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), _ptr(gates), float(cap), float(q_scale),
+            pointer, stride, _ptr(state_slots), _ptr(row_start), _ptr(row_len), _ptr(row_ctx), _ptr(coefficients), _ptr(out), _ptr(below),
+            rows, heads, dim, value_dim, _stream()), "matrix_memory")
+
+    def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim, gate_activation="silu", below=None, floor=0.0):
         n = x.shape[0]
+        if gate_activation not in self.GATE_ACTIVATIONS:
+            raise ValueError(f"the heads' gate is one of {self.GATE_ACTIVATIONS}, not {gate_activation!r}")
+        if below is not None:
+            _check(below, "below", torch.float32, (n, heads, 2))
         _check(x, "x", torch.float32, (n, heads * value_dim))
         _check(weight, "weight", torch.float32, (heads * value_dim if weight_per_channel else value_dim,))
         _check(out, "out", None, (n, heads * value_dim))
@@ -1147,7 +1221,7 @@ class HipOps(KernelNamespace):
             raise ValueError(f"gate must be a view [{n}, {heads * value_dim}] of {out.dtype} on the GPU with unit stride along a row")
         _launched(self._part_library("recurrent").lsa_heads_norm_gate(
             _code(out), _ptr(x), _ptr(weight), 1 if weight_per_channel else 0, float(eps), gate.data_ptr(), gate.stride(0), _ptr(out),
-            n, heads, value_dim, _stream()), "heads_norm_gate")
+            n, heads, value_dim, self.GATE_ACTIVATIONS.index(gate_activation), _ptr(below), float(floor), _stream()), "heads_norm_gate")
 
     def scaled_sum(self, x, x_scale, y, y_scale, out):
         _check(x, "x")

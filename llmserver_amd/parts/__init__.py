@@ -1,17 +1,18 @@
 from .attention import AttentionNames, AttentionPlan, AttentionTuning, GQAttention, TileLaunchCost, build_attention_plan, group_tiling
 from .base import (INT_TABLE, MATRIX, VECTOR, Block, FeedForward, Mixer, Norm, PagedAndStateSpec, PagedKVSpec, ParamSpec, Part,
                    PositionEncoding, StateSpec)
-from .block import DepthAverage, PostNormBlock, PreNormBlock, SandwichBlock
+from .block import DepthAverage, HyperConnection, MultiStreamBlock, PostNormBlock, PreNormBlock, SandwichBlock
 from .conv import ShortConvolution
 from .embedding import NormedTokenEmbedding, TokenEmbedding
 from .experts import RoutedExperts
 from .kernel_namespace import KernelNamespace
 from .latent_attention import LatentAttention, LatentAttentionNames
 from .linear import Linear
-from .mlp import GatedMLP, GatedMLPNames
-from .norm import RMSNorm
+from .mlp import GatedMLP, GatedMLPNames, PlainMLP
+from .norm import RMSNorm, StreamReadNorm
 from .parallel import ParallelMixers, ScaledPair
-from .recurrent import GatedLinearAttention, GatedLinearAttentionNames, TimeMixing, TimeMixingNames, TokenShift
+from .recurrent import (GatedLinearAttention, GatedLinearAttentionNames, MatrixMemory, MatrixMemoryNames, TimeMixing, TimeMixingNames,
+                        TokenShift)
 from .rope import NoPosition, PairedRotaryPosition, RotaryPosition
 
 __all__ = ["KernelNamespace", "AttentionNames", "AttentionTuning", "TileLaunchCost", "GatedMLPNames", "AttentionPlan", "GQAttention", "build_attention_plan", "group_tiling", "INT_TABLE", "MATRIX", "VECTOR",
@@ -19,4 +20,5 @@ __all__ = ["KernelNamespace", "AttentionNames", "AttentionTuning", "TileLaunchCo
            "StateSpec", "PreNormBlock", "TokenEmbedding", "Linear", "GatedMLP", "RMSNorm", "NoPosition",
            "RotaryPosition", "PairedRotaryPosition", "PagedAndStateSpec", "DepthAverage", "PostNormBlock", "ShortConvolution",
            "NormedTokenEmbedding", "RoutedExperts", "LatentAttention", "LatentAttentionNames", "SandwichBlock", "ParallelMixers",
-           "ScaledPair", "GatedLinearAttention", "GatedLinearAttentionNames", "TimeMixing", "TimeMixingNames", "TokenShift"]
+           "ScaledPair", "HyperConnection", "MultiStreamBlock", "PlainMLP", "StreamReadNorm", "MatrixMemory", "MatrixMemoryNames",
+           "GatedLinearAttention", "GatedLinearAttentionNames", "TimeMixing", "TimeMixingNames", "TokenShift"]

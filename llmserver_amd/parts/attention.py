@@ -24,6 +24,7 @@ import dataclasses
 from typing import Optional, Tuple
 
 import numpy as np
+import torch
 
 from .base import VECTOR, Mixer, PagedKVSpec, ParamSpec, PositionEncoding
 from .kernel_namespace import tuning_of
@@ -450,12 +451,15 @@ class GQAttention(Mixer):
                  qk_norm_eps: Optional[float] = None, bias: bool = False, out_bias: Optional[bool] = None,
                  window: Optional[int] = None, scale: Optional[float] = None, names: AttentionNames = AttentionNames(),
                  sinks: Optional[str] = None, softcap: Optional[float] = None, value_dim: Optional[int] = None,
-                 bare_names: bool = False):
+                 bare_names: bool = False, bias_suffix: str = "", values_are_keys: bool = False):
         """``sinks``: the checkpoint name of a float vector ``[n_heads]`` whose exponentials join the softmax's
         denominators (one term per head, without a key or a value), or None.  ``softcap``: scores become
         ``softcap * tanh(score / softcap)`` (after the scale, before the mask), or None.  ``value_dim``: the size of a
         head's values if it is not the size of its queries and keys.  ``bare_names``: the names are the tensors' whole
-        names (no ``.weight`` behind them).
+        names (no ``.weight`` behind them; a bias is then named ``<matrix><bias_suffix>``).  ``values_are_keys``: there is
+        no value projection; a token's values are its keys as projected (bias included), before norm and rotation.
+        ``names.qkv`` then names queries and keys only, and the stacked matrix gets the keys' rows a second time in
+        the values' place when the tensors have been loaded, so every kernel sees queries, keys and values as usual.
 
         A position encoding that turns neighbouring dimensions together (``pairing == "neighbours"``), a rotation of a
         part of the head, values of another size than the keys, and head sizes that are no multiple of 16 go the general
@@ -470,11 +474,12 @@ class GQAttention(Mixer):
         self.general = paired or self.value_dim != head_dim or head_dim % 16 != 0 or \
             (position.rotary_dim is not None and position.rotary_dim != head_dim)
         if self.general:
-            if position.rotary_dim is not None and (not paired or position.rotary_dim > head_dim):
-                raise ValueError(f"the position encoding rotates {position.rotary_dim} of a head's {head_dim} dimensions; a rotation of a "
-                                 "part of the head is built for encodings that turn neighbouring dimensions together")
-            if bias:
-                raise ValueError("the general way of preparing queries, keys and values takes projections without biases")
+            if position.rotary_dim is not None and position.rotary_dim > head_dim:
+                raise ValueError(f"the position encoding rotates {position.rotary_dim} dimensions, a head has {head_dim}")
+        self.pairing = "neighbours" if paired else "halves"
+        self.values_are_keys = bool(values_are_keys)
+        if values_are_keys and (self.value_dim != head_dim or len(names.qkv) != 2):
+            raise ValueError("values that are the keys have the keys' size, and the checkpoint names queries and keys: two tensors")
         self.row = -(-max(head_dim, self.value_dim) // 16) * 16      # a head as the attention kernels and the pages see it
         self.position = position
         self.qk_norm_eps = qk_norm_eps
@@ -483,11 +488,14 @@ class GQAttention(Mixer):
         self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
         q_rows, k_rows, v_rows = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * self.value_dim
         stacked = {3: (q_rows, k_rows, v_rows), 2: (q_rows, k_rows + v_rows), 1: (q_rows + k_rows + v_rows,)}
+        if values_are_keys:
+            stacked = {2: (q_rows, k_rows)}
         if len(names.qkv) not in stacked:
             raise ValueError(f"queries, keys and values come in one, two or three checkpoint tensors, not {len(names.qkv)}")
         self.names, self.bare_names = names, bare_names
-        self.qkv = Linear(width, names.qkv, stacked[len(names.qkv)], bias, bare_names=bare_names)
-        self.o = Linear(n_heads * self.value_dim, (names.out,), (width,), bias if out_bias is None else out_bias, bare_names=bare_names)
+        self.qkv = Linear(width, names.qkv, stacked[len(names.qkv)], bias, bare_names=bare_names, bias_suffix=bias_suffix)
+        self.o = Linear(n_heads * self.value_dim, (names.out,), (width,), bias if out_bias is None else out_bias, bare_names=bare_names,
+                        bias_suffix=bias_suffix)
         self.q_norm_weight = None
         self.k_norm_weight = None
         self.sinks_name, self.sinks = sinks, None
@@ -517,9 +525,9 @@ class GQAttention(Mixer):
             self.q_norm_weight = tensor
         elif owner == self.names.k_norm:
             self.k_norm_weight = tensor
-        elif owner == self.names.out:
+        elif owner == self.names.out or self.o.owns(name):
             self.o.assign(name, tensor)
-        elif owner in self.names.qkv:
+        elif owner in self.names.qkv or self.qkv.owns(name):
             self.qkv.assign(name, tensor)
         else:
             raise KeyError(name)
@@ -527,6 +535,15 @@ class GQAttention(Mixer):
     def finalize(self):
         self.qkv.finalize()
         self.o.finalize()
+        if self.values_are_keys and self.qkv.weight.shape[0] == (self.n_heads + self.n_kv_heads) * self.head_dim:
+            # the keys' rows once more, where the kernels look for the values
+            from_keys = self.n_heads * self.head_dim
+            self.qkv.weight = torch.cat([self.qkv.weight, self.qkv.weight[from_keys:]], dim=0).contiguous()
+            for name in ("bias", "bias_rounded"):
+                vector = getattr(self.qkv, name)
+                if vector is not None:
+                    setattr(self.qkv, name, torch.cat([vector, vector[from_keys:]], dim=0).contiguous())
+            self.qkv.out_features = self.qkv.weight.shape[0]
         if self.row != self.value_dim:
             # The attention kernels leave a head's result in a row of `row` numbers, zeros behind the values: the output
             # projection reads those rows as they are, through columns of zeros.
@@ -564,7 +581,8 @@ class GQAttention(Mixer):
         q = ctx.empty((n, self.n_heads * self.row))
         ctx.ops.qkv_prepare(qkv, cache.keys, cache.values, table, ctx.token_row, ctx.positions, self.q_norm_weight, self.k_norm_weight,
                             self.qk_norm_eps if self.qk_norm_eps is not None else 0.0, self.position.cos_sin(ctx), cache.page_size,
-                            self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim, q, cache.writable)
+                            self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim, q, cache.writable,
+                            **({"pairing": "halves"} if self.pairing == "halves" and self.position.rotary_dim is not None else {}))
         out = ctx.empty((n, self.n_heads * self.row))
         extra = {}
         if self.sinks is not None:

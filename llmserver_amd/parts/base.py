@@ -25,7 +25,7 @@ class ParamSpec:
     """One checkpoint tensor of a part: its shape, how it is stored and how random weights draw it."""
     shape: Tuple[int, ...]
     role: str = MATRIX
-    init: str = "normal"          # "normal" | "norm" | "bias" | "zeros"
+    init: str = "normal"          # "normal" | "norm" | "bias" | "zeros" | "identity"
     optional: bool = False         # may be absent from the checkpoint
     # The share of the tensor that one token's pass uses: 1 for a dense layer's matrix, k/n for one of n experts of
     # which a token chooses k, 0 for a table of which a token reads a row.  (What a step costs is summed from this.)

@@ -261,3 +261,127 @@ class SandwichBlock(Block):
     def _same_kind(following):
         """The next block's first norm, if its kernel can be folded in here (a plain RMS norm of the stream)."""
         return following if following is not None and hasattr(following, "weight") and hasattr(following, "eps") else None
+
+
+class HyperConnection(Part):
+    """How one sublayer is connected to ``streams`` residual streams ``x_1 .. x_S``.  It reads ``sum_s read[s] * x_s``; its
+    result ``y`` changes all streams at once, from the old ones: ``x_t <- sum_s mix[s, t] * x_s + mult * write[t] * y``
+    (``mix`` indexed [from, to]).  ``learned``: ``read``, ``write`` and ``mix`` are checkpoint tensors (``names``); not
+    learned, they are ones and the identity, which is the plain residual sum ``x <- x + mult * y`` on one stream."""
+
+    def __init__(self, streams: int, mult: float = 1.0, learned: bool = True, names=("in", "out", "mix")):
+        self.streams, self.mult, self.learned, self.names = int(streams), float(mult), bool(learned), tuple(names)
+        self.read = self.write = self.mix = None        # float32 [S], [S] (times mult), [S, S]
+
+    def param_specs(self):
+        if not self.learned:
+            return {}
+        read, write, mix = self.names
+        return {read: ParamSpec((self.streams,), VECTOR, "norm"), write: ParamSpec((self.streams,), VECTOR, "norm"),
+                mix: ParamSpec((self.streams, self.streams), VECTOR, "identity")}
+
+    def assign(self, name, tensor):
+        read, write, mix = self.names
+        if name == read:
+            self.read = tensor
+        elif name == write:
+            self.write = tensor
+        elif name == mix:
+            self.mix = tensor
+        else:
+            raise KeyError(name)
+
+    def settle(self, like: torch.Tensor) -> None:
+        """Once all tensors are there (``like``: any float32 tensor of the block, for its device)."""
+        if not self.learned:
+            self.read, self.write = like.new_ones((self.streams,)), like.new_ones((self.streams,))
+            self.mix = torch.eye(self.streams, device=like.device, dtype=like.dtype)
+        self.write = (self.write * self.mult).contiguous()
+        self.read, self.mix = self.read.contiguous(), self.mix.contiguous()
+
+
+class MultiStreamBlock(Block):
+    """Pre-norm sublayers over several residual streams kept in 32-bit, ``[streams, T, W]``: each sublayer reads a
+    weighted sum of the streams under its norm and writes its result, times a constant, back into all of them through
+    its :class:`HyperConnection`; ``ffn`` may be None.  With one stream and connections that are not learned this is
+    the plain ``x <- x + mult * sublayer(norm(x))``.  The update behind a sublayer and the read and norm in front of the
+    next one (the next block's, if it is of this kind) are one kernel (``ops.streams_update``).
+
+    ``mixer_norm`` / ``ffn_norm``: :class:`~llmserver_amd.parts.norm.StreamReadNorm`; ``names``: the checkpoint's names of
+    the mixer's norm, the mixer, the feed-forward's norm, the feed-forward and the two connections."""
+    takes_following = True
+
+    def __init__(self, mixer_norm, mixer: Mixer, mixer_connection: HyperConnection, ffn_norm=None, ffn=None, ffn_connection=None,
+                 names=("norm1", "mix", "norm2", "mlp", "hc1", "hc2")):
+        self.mixer_norm, self.mixer, self.mixer_connection = mixer_norm, mixer, mixer_connection
+        self.ffn_norm, self.ffn, self.ffn_connection = ffn_norm, ffn, ffn_connection
+        self.names = tuple(names)
+        self.streams = mixer_connection.streams
+
+    def _parts(self):
+        norm1, mix, norm2, mlp, hc1, hc2 = self.names
+        parts = {norm1: self.mixer_norm, mix: self.mixer, hc1: self.mixer_connection}
+        if self.ffn is not None:
+            parts.update({norm2: self.ffn_norm, mlp: self.ffn, hc2: self.ffn_connection})
+        return parts
+
+    def param_specs(self):
+        return {f"{prefix}.{name}" if name else prefix: spec for prefix, part in self._parts().items()
+                for name, spec in part.param_specs().items()}
+
+    def assign(self, name, tensor):
+        parts = self._parts()
+        if name in parts:                                   # the part's name is the tensor's
+            parts[name].assign("", tensor)
+            return
+        prefix, rest = name.split(".", 1)
+        parts[prefix].assign(rest, tensor)
+
+    def finalize(self):
+        self.mixer_connection.settle(self.mixer_norm.weight)
+        self.mixer_norm.read_weights = self.mixer_connection.read
+        if self.ffn is not None:
+            self.ffn_connection.settle(self.ffn_norm.weight)
+            self.ffn_norm.read_weights = self.ffn_connection.read
+        for part in self._parts().values():
+            part.finalize()
+
+    def entry_norm(self):
+        return self.mixer_norm
+
+    def _update(self, ctx, streams, result, connection, following):
+        """The streams behind a sublayer (updated where they lie) and, if ``following`` is given, what the next sublayer
+        reads from them under its norm, in the compute type."""
+        normed = ctx.empty(streams.shape[1:]) if following is not None else None
+        ctx.ops.streams_update(streams, result, connection.mix, connection.write,
+                               following.read_weights if following is not None else None,
+                               following.weight if following is not None else None,
+                               following.eps if following is not None else 0.0, normed)
+        return streams, normed
+
+    def _same_kind(self, following):
+        """The next block's first norm, if it reads as many streams as this block keeps."""
+        from .norm import StreamReadNorm
+        return following if isinstance(following, StreamReadNorm) and following.streams == self.streams \
+            and following.read_weights is not None else None
+
+    def forward(self, resid, delta, ctx, cache, following=None):
+        """``delta``: None, or a :class:`StreamUpdate` whose ``normed`` rows are what this block's mixer reads (the block
+        before was told this block's first norm as its ``following`` and has carried it out)."""
+        streams, h = resid, None
+        if isinstance(delta, StreamUpdate):
+            streams = delta.resid
+            h = delta.normed if delta.norm is self.mixer_norm else None
+        elif delta is not None:
+            raise ValueError("this block takes streams to which everything has been added")
+        if h is None:
+            h = self.mixer_norm.add_norm(streams, None, ctx)
+        mixed = self.mixer.forward(h, ctx, cache)
+        following = self._same_kind(following)
+        if self.ffn is None:
+            streams, normed = self._update(ctx, streams, mixed, self.mixer_connection, following)
+        else:
+            streams, h = self._update(ctx, streams, mixed, self.mixer_connection, self.ffn_norm)
+            fed = self.ffn.forward(h, ctx)
+            streams, normed = self._update(ctx, streams, fed, self.ffn_connection, following)
+        return streams, (StreamUpdate(following, streams, normed=normed) if normed is not None else None)

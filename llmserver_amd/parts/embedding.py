@@ -1,4 +1,5 @@
-"""Token embedding lookup ``h0 = E[ids]`` without scaling (utils/model.py:56-59,110)."""
+"""Token embedding lookup ``h0 = E[ids]`` (utils/model.py:56-59,110), optionally times a constant and into several
+residual streams at once."""
 from __future__ import annotations
 
 import torch
@@ -8,10 +9,15 @@ from .base import MATRIX, ParamSpec, Part
 
 class TokenEmbedding(Part):
     """``tensor``: the table's name below the part's own ("" if the part's name is the tensor's).  ``wide``: the rows
-    start a residual stream that is kept in 32-bit whatever the type of the table."""
+    start a residual stream that is kept in 32-bit whatever the type of the table.  ``scale``: what a wide row is
+    multiplied by (in 32-bit; the table itself stays as stored, so a head that shares it reads it unscaled).
+    ``streams``: a wide stream starts as this many equal copies ``[streams, T, W]`` (0: one stream ``[T, W]``)."""
 
-    def __init__(self, vocab: int, width: int, tensor: str = "weight", wide: bool = False):
+    def __init__(self, vocab: int, width: int, tensor: str = "weight", wide: bool = False, scale: float = 1.0, streams: int = 0):
+        if (scale != 1.0 or streams) and not wide:
+            raise ValueError("a scaled embedding, and one that starts several streams, starts a 32-bit stream (wide=True)")
         self.vocab, self.width, self.tensor, self.wide = vocab, width, tensor, wide
+        self.scale, self.streams = float(scale), int(streams)
         self.weight = None
 
     def param_specs(self):
@@ -23,8 +29,12 @@ class TokenEmbedding(Part):
 
     def forward(self, token_ids, ctx):
         if self.wide:
-            out = ctx.empty((token_ids.shape[0], self.width), dtype=torch.float32)
-            ctx.ops.embedding_wide(self.weight, token_ids, out)
+            shape = (token_ids.shape[0], self.width)
+            out = ctx.empty((self.streams, *shape) if self.streams else shape, dtype=torch.float32)
+            if self.scale != 1.0 or self.streams:
+                ctx.ops.embedding_wide(self.weight, token_ids, out, scale=self.scale)
+            else:
+                ctx.ops.embedding_wide(self.weight, token_ids, out)
             return out
         out = ctx.empty((token_ids.shape[0], self.width))
         ctx.ops.embedding(self.weight, token_ids, out)

@@ -52,10 +52,11 @@ class KernelNamespace:
         raise NotImplementedError
 
     def qkv_prepare(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
-                    n_q, n_kv, dim, value_dim, out_q, write_cache=True):
+                    n_q, n_kv, dim, value_dim, out_q, write_cache=True, pairing="neighbours"):
         """``qkv [T, n_q * dim + n_kv * dim + n_kv * value_dim]``.  Per head, queries and keys are RMS-normed over ``dim``
         (``q_weight`` / ``k_weight [dim]`` float32, or both None: no norm), then the first ``2 * pairs`` dimensions turn
-        in neighbouring pairs (2i, 2i+1) by ``cos_sin [T, 2 * pairs]`` (cosines, then sines; None: no rotation).  With
+        in neighbouring pairs (2i, 2i+1) or, with ``pairing="halves"``, in pairs (i, i + pairs), by ``cos_sin [T, 2 * pairs]``
+        (cosines, then sines; None: no rotation).  With
         ``D`` the pages' head size: ``out_q [T, n_q * D]`` gets the query rows, zeros behind ``dim``; with ``write_cache``,
         ``keys [pages, n_kv, page_size, D]`` get the key rows and ``values [pages, n_kv, D, page_size]`` the value rows
         (zeros behind ``dim`` / ``value_dim``) at every token's place."""
@@ -92,9 +93,40 @@ class KernelNamespace:
         the state after the row's last token is stored back."""
         raise NotImplementedError
 
-    def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim):
-        """``out[t, h, :] = x[t, h, :] / rms(x[t, h, :]) * w * silu(gate[t, h, :])``; ``x`` float32, ``w = weight [value_dim]``
-        shared by the heads or, with ``weight_per_channel``, ``weight [heads * value_dim]``; ``gate`` a view like ``out``."""
+    def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim, gate_activation="silu", below=None, floor=0.0):
+        """``out[t, h, :] = x'[t, h, :] / rms(x'[t, h, :]) * w * act(gate[t, h, :])``; ``x`` float32, ``w = weight [value_dim]``
+        shared by the heads or, with ``weight_per_channel``, ``weight [heads * value_dim]``; ``gate`` a view like ``out``;
+        ``act``: ``"silu"`` or ``"sigmoid"``.  ``x' = x``, or, with ``below [T, heads, 2]`` (float32):
+        ``x / (max(|below[..., 0]|, below[..., 1]) + floor)``, a matrix memory's read-out under its normaliser."""
+        raise NotImplementedError
+
+    def matrix_memory(self, q, k, v, gates, cap, q_scale, state, state_slots, row_start, row_len, row_ctx, out, below, coefficients,
+                      heads, dim, value_dim):
+        """A matrix memory with exponential gates, per row (request) and head over the row's tokens in order, all float32.
+        ``gates [T, 2 * heads]``: the input gates' logits, then the forget gates'.  ``i = cap * tanh(z_i / cap)``,
+        ``f = logsigmoid(cap * tanh(z_f / cap))``, ``m_t = max(f + m_(t-1), i)``, ``keep = exp(f + m_(t-1) - m_t)``,
+        ``take = exp(i - m_t)``; ``S_t = keep S_(t-1) + take k_t v_t^T``, ``n_t = keep n_(t-1) + take k_t``.
+        ``out [T, heads * value_dim] = S_t^T (q_t * q_scale)`` (the numerators only), ``below [T, heads, 2] =
+        (n_t . (q_t * q_scale), exp(-m_t))``, ``coefficients [T, heads, 2]`` scratch (keep, take).  ``q, k [T, heads * dim]``,
+        ``v [T, heads * value_dim]`` (views with unit stride along a row).  ``state[slot]``: ``S [heads, dim, value_dim]``,
+        then ``n [heads, dim]``, then ``m [heads]``; a row whose first token stands at position 0 starts from zeros whatever
+        the slot holds; the state after the row's last token is stored back."""
+        raise NotImplementedError
+
+    # Several residual streams in 32-bit.
+    def streams_read(self, streams, read, weight, eps, out, rows=None):
+        """``out = rmsnorm(sum_s read[s] * streams[s, rows]) * weight``; ``streams [S, T, W]`` float32, ``rows`` int32 or None
+        (all); ``out`` of any type."""
+        raise NotImplementedError
+
+    def streams_update(self, streams, y, mix, write, next_read=None, next_weight=None, next_eps=0.0, normed=None):
+        """Where they lie, all streams at once from the old ones: ``streams[t] <- sum_s mix[s, t] * streams[s] + write[t] * y``
+        (``y [T, W]`` of any type).  With ``next_read``: ``normed = rmsnorm(sum_t next_read[t] * streams[t]) * next_weight``
+        of the new streams (eps ``next_eps``, any type)."""
+        raise NotImplementedError
+
+    def activation_(self, x, activation):
+        """``x = act(x)`` where it lies, in 32-bit, rounded once: ``"relu2"`` (``max(x, 0)^2``), ``"gelu_tanh"``, ``"silu"``."""
         raise NotImplementedError
 
     def scaled_sum(self, x, x_scale, y, y_scale, out):
@@ -105,8 +137,8 @@ class KernelNamespace:
         """``out [T, W]`` float32 ``= rmsnorm(table[token_ids]) * weight``."""
         raise NotImplementedError
 
-    def embedding_wide(self, table, token_ids, out):
-        """``out [T, W]`` float32 ``= table[token_ids]``."""
+    def embedding_wide(self, table, token_ids, out, scale=1.0):
+        """``out [T, W]`` float32 ``= table[token_ids] * scale``; an ``out [S, T, W]`` gets the rows ``S`` times."""
         raise NotImplementedError
 
     def norm_add_norm(self, x, y, weight, eps, out, next_weight=None, next_eps=0.0, normed=None, y2=None, scales=None):
@@ -146,8 +178,9 @@ class KernelNamespace:
         ``q_latent`` None and ``up_keys [heads, dim, rank]`` given: ``q_latent[h, t] = q_plain[t, h] @ up_keys[h]`` is made here."""
         raise NotImplementedError
 
-    def gate_heads(self, y, proj, gate_column, out, mixed=None, up_values=None):
-        """``out[t, h * v + j] = y[h, t, j] * sigmoid(proj[t, gate_column + h])`` (``gate_column`` < 0: no gate).  ``y`` None and
+    def gate_heads(self, y, proj, gate_column, out, mixed=None, up_values=None, per_channel=False):
+        """``out[t, h * v + j] = y[h, t, j] * sigmoid(proj[t, gate_column + h])`` (``gate_column`` < 0: no gate; ``per_channel``:
+        a gate for every channel, ``proj[t, gate_column + h * v + j]``).  ``y`` None and
         ``mixed [T, heads * row]``, ``up_values [heads, rank, v]`` given: ``y[h, t] = mixed[t, h, :rank] @ up_values[h]`` is made here."""
         raise NotImplementedError
 

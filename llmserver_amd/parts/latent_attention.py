@@ -9,7 +9,8 @@ attention kernel sees one key-value head that all query heads share, with the ca
 row is padded with zeros to the next head size the attention kernels take.
 
 The softmax's denominator may hold one more term per head (``exp(sink)``, no key, no value), and every head's output
-may pass a sigmoid gate computed from the mixer's input.
+may pass a sigmoid gate computed from the mixer's input: one gate a head, or one for every channel of every head.  A
+window bounds the keys a query sees to the last ``window`` positions; pages behind it go back to the pool.
 """
 from __future__ import annotations
 
@@ -44,19 +45,24 @@ class LatentAttention(Mixer):
     graph_safe = True
 
     def __init__(self, width: int, n_heads: int, dim: int, rot_dim: int, value_dim: int, rank: int, position: PositionEncoding,
-                 scale: float, norm_eps: float, names: LatentAttentionNames = LatentAttentionNames()):
+                 scale: float, norm_eps: float, names: LatentAttentionNames = LatentAttentionNames(), window: Optional[int] = None,
+                 gate_per_channel: bool = False):
+        """``window``: a query sees itself and the ``window - 1`` positions before it (None: all).  ``gate_per_channel``:
+        the gate's projection has a row for every channel of every head's values instead of one a head."""
         if getattr(position, "pairing", None) != "neighbours":
             raise ValueError("this mixer's kernels turn neighbouring dimensions together; it takes a PairedRotaryPosition")
         if position.rotary_dim is None or position.rotary_dim > rot_dim or position.rotary_dim % 2:
             raise ValueError(f"the position encoding turns {position.rotary_dim} dimensions, the rotated part has {rot_dim}")
         self.width, self.n_heads, self.dim, self.rot_dim, self.value_dim, self.rank = width, n_heads, dim, rot_dim, value_dim, rank
         self.position, self.scale, self.norm_eps, self.names = position, float(scale), float(norm_eps), names
+        self.window = int(window) if window else None
+        self.gate_per_channel = bool(gate_per_channel) and names.gate is not None
         self.row = padded_head(rank + rot_dim)       # the cached row, as wide as a head of the attention kernels
         self.q_width = n_heads * (dim + rot_dim)
         pieces, sizes = [names.q, names.down], [self.q_width, rank + rot_dim]
         if names.gate is not None:
             pieces.append(names.gate)
-            sizes.append(n_heads)
+            sizes.append(n_heads * value_dim if self.gate_per_channel else n_heads)
         self.proj = Linear(width, pieces, sizes, bare_names=True)      # queries, latent and shared key part, gates: one product
         self.o = Linear(n_heads * value_dim, (names.out,), (width,), bare_names=True)
         self.down_norm_weight = None
@@ -66,7 +72,7 @@ class LatentAttention(Mixer):
         self.up_values = None      # [heads, rank, value_dim]: out = latent_sum @ up_values[head]
 
     def cache_spec(self):
-        return PagedKVSpec(1, self.row, None)
+        return PagedKVSpec(1, self.row, self.window)
 
     def param_specs(self):
         specs = {**self.proj.param_specs(), **self.o.param_specs()}
@@ -103,7 +109,7 @@ class LatentAttention(Mixer):
 
     def plan_key(self):
         # (the row's width is part of it: the plan is cut for the kernels of that head size)
-        return ("paged_attention", self.n_heads, 1, None, self.row)
+        return ("paged_attention", self.n_heads, 1, self.window, self.row)
 
     def graph_shape(self, rows: int, longest_context: int):
         return "short contexts" if longest_context <= SHORT_CONTEXT else None
@@ -114,11 +120,14 @@ class LatentAttention(Mixer):
     def mixing_flops(self, new_tokens: int, context: int) -> float:
         """Scores over ``rank + rot_dim`` and weighted latents over ``rank`` dimensions per head, query and visible key."""
         first = context - new_tokens
-        pairs = new_tokens * first + new_tokens * (new_tokens + 1) // 2
+        if self.window is None:
+            pairs = new_tokens * first + new_tokens * (new_tokens + 1) // 2
+        else:
+            pairs = sum(min(position + 1, self.window) for position in range(first, context))
         return 2.0 * self.n_heads * (2 * self.rank + self.rot_dim) * pairs
 
     def prepare(self, ctx):
-        stage_attention_plan(ctx, self.plan_key(), self.n_heads, 1, self.row, None, self.graph_shape)
+        stage_attention_plan(ctx, self.plan_key(), self.n_heads, 1, self.row, self.window, self.graph_shape)
 
     def forward(self, x, ctx, cache):
         ops = ctx.ops
@@ -138,13 +147,14 @@ class LatentAttention(Mixer):
         mixed = ctx.empty((n, self.n_heads * self.row))
         extra = {"sinks": self.sinks} if self.sinks is not None else {}
         ops.paged_attention(q, mixed, cache.keys, cache.values, table, ctx.row_start, ctx.row_len, ctx.row_ctx,
-                            ctx.get_plan(self.plan_key()), self.scale, None, cache.page_size, self.n_heads, 1, self.row, ctx, **extra)
+                            ctx.get_plan(self.plan_key()), self.scale, self.window, cache.page_size, self.n_heads, 1, self.row, ctx, **extra)
         gated = ctx.empty((n, self.n_heads * self.value_dim))
         # (without gates the same kernel only brings the heads back beside each other: a gate column of -1 says so)
         gate_column = self.q_width + self.rank + self.rot_dim if self.names.gate is not None else -1
+        wide = {"per_channel": True} if self.gate_per_channel else {}
         if inside:
-            ops.gate_heads(None, proj, gate_column, gated, mixed=mixed, up_values=self.up_values)
+            ops.gate_heads(None, proj, gate_column, gated, mixed=mixed, up_values=self.up_values, **wide)
         else:
             latent = mixed.view(n, self.n_heads, self.row)[:, :, :self.rank].transpose(0, 1)
-            ops.gate_heads(torch.bmm(latent, self.up_values), proj, gate_column, gated)      # [heads, T, value_dim]
+            ops.gate_heads(torch.bmm(latent, self.up_values), proj, gate_column, gated, **wide)      # [heads, T, value_dim]
         return self.o.forward(gated, ctx)

@@ -19,14 +19,16 @@ class Linear(Part):
     """One GEMM over one or several stacked checkpoint matrices.
 
     ``names``/``out_features`` list the stacked pieces in output order, e.g. ``("q_proj",
-    "k_proj", "v_proj")``.  Tensor names are ``<piece>.weight`` and ``<piece>.bias``.
+    "k_proj", "v_proj")``.  Tensor names are ``<piece>.weight`` and ``<piece>.bias``; with ``bare_names`` a piece's
+    name is its matrix's whole name, and its bias, if it has one, is that name with ``bias_suffix`` behind it.
     """
 
     def __init__(self, in_features: int, pieces: Sequence[str], out_features: Sequence[int], bias: bool = False,
-                 out_float32: bool = False, bare_names: bool = False):
-        if bare_names and bias:
-            raise ValueError("a piece whose name is the tensor's has no place for a bias")
+                 out_float32: bool = False, bare_names: bool = False, bias_suffix: str = ""):
+        if bare_names and bias and not bias_suffix:
+            raise ValueError("a piece whose name is the tensor's has no place for a bias unless bias_suffix names one")
         self.bare_names = bare_names        # the pieces' names are the tensors' names (no ".weight" behind them)
+        self.bias_suffix = bias_suffix
         self.in_features = in_features
         self.pieces = tuple(pieces)
         self.piece_out = tuple(out_features)
@@ -44,12 +46,19 @@ class Linear(Part):
         for piece, n in zip(self.pieces, self.piece_out):
             specs[piece if self.bare_names else f"{piece}.weight"] = ParamSpec((n, self.in_features), MATRIX, "normal")
             if self.has_bias:
-                specs[f"{piece}.bias"] = ParamSpec((n,), VECTOR, "bias")
+                specs[piece + self.bias_suffix if self.bare_names else f"{piece}.bias"] = ParamSpec((n,), VECTOR, "bias")
         return specs
+
+    def owns(self, name: str) -> bool:
+        """Whether ``name`` is one of this projection's tensors."""
+        return name in self.param_specs()
 
     def assign(self, name, tensor):
         if self.bare_names:
-            self._w[name] = tensor
+            if self.has_bias and name not in self.pieces and name.endswith(self.bias_suffix):
+                self._b[name[:-len(self.bias_suffix)]] = tensor
+            else:
+                self._w[name] = tensor
             return
         piece, kind = name.rsplit(".", 1)
         (self._w if kind == "weight" else self._b)[piece] = tensor

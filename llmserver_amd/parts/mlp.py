@@ -1,4 +1,5 @@
-"""Gated feed-forward ``down(act(gate(x)) * up(x))``; ``act`` is SiLU or the tanh form of GELU.
+"""Gated feed-forward ``down(act(gate(x)) * up(x))``; ``act`` is SiLU or the tanh form of GELU.  And the plain one,
+``down(act(up(x)))``, whose ``act`` may also be the square of the rectifier.
 
 Gate and up are one stacked product, gate first (utils/layers.py:194-218;
 utils/fused_ops.py:59-61, 80-88).  Sigmoid and the product run in 32-bit inside
@@ -83,3 +84,39 @@ class GatedMLP(FeedForward):
         hidden = ctx.empty((gate_up.shape[0], self.intermediate))
         ops.swiglu(gate_up, hidden, activation=self.activation)
         return self.down.forward(hidden, ctx, sink=sink)
+
+
+class PlainMLP(FeedForward):
+    """``down(act(up(x)))`` without a gate.  ``activation``: ``"relu2"`` (``max(z, 0)^2``), ``"gelu_tanh"`` or ``"silu"``,
+    computed in 32-bit and stored over the up projection's result.  ``names``: the checkpoint names of the two matrices."""
+
+    ACTIVATIONS = ("relu2", "gelu_tanh", "silu")
+
+    def __init__(self, width: int, intermediate: int, activation: str = "relu2", names: Tuple[str, str] = ("up", "down"),
+                 bare_names: bool = False):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"Unsupported activation {activation!r}; supported: {list(self.ACTIVATIONS)}")
+        self.width, self.intermediate, self.activation = width, intermediate, activation
+        self.names, self.bare_names = tuple(names), bare_names
+        self.up = Linear(width, (names[0],), (intermediate,), bare_names=bare_names)
+        self.down = Linear(intermediate, (names[1],), (width,), bare_names=bare_names)
+
+    def param_specs(self):
+        return {**self.up.param_specs(), **self.down.param_specs()}
+
+    def assign(self, name, tensor):
+        if self.up.owns(name):
+            self.up.assign(name, tensor)
+        elif self.down.owns(name):
+            self.down.assign(name, tensor)
+        else:
+            raise KeyError(name)
+
+    def finalize(self):
+        self.up.finalize()
+        self.down.finalize()
+
+    def forward(self, x, ctx):
+        hidden = self.up.forward(x, ctx)
+        ctx.ops.activation_(hidden, self.activation)
+        return self.down.forward(hidden, ctx)

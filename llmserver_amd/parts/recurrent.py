@@ -7,6 +7,10 @@ Two readings of the state are built on one kernel (``ops.linear_recurrence``):
 * ``bonus [heads, dim]``: ``o_t = (S_(t-1) + diag(bonus) k_t v_t^T)^T q_t``, then the state moves on (the token itself
   enters the output through the bonus only).
 
+A third reading, on a kernel of its own (``ops.matrix_memory``), is the matrix memory with exponential gates
+(:class:`MatrixMemory`): one input and one forget gate a head, kept in range by a running maximum of their logarithms,
+and a normaliser vector beside the matrix.
+
 The decay comes from a low-rank map of the mixer's input whose result stays in 32-bit; how it becomes a number in
 (0, 1) is the kernel's ``decay`` mode: ``"sigmoid_root"`` (``sigmoid(z)^(1/tau)``) or ``"double_exp"`` (``exp(-exp(z))``).
 The state ``[heads, dim, vdim]`` is float32, one slot per live request, zeros before a sequence's first token, and it is
@@ -265,4 +269,94 @@ class TimeMixing(Mixer):
                               ctx.state_slots, ctx.row_start, ctx.row_len, ctx.row_ctx, mixed, self.heads, self.dim, self.dim)
         gated = ctx.empty((n, inner))
         ops.heads_norm_gate(mixed, self.norm_weight, True, self.norm_eps, four[3], gated, self.heads, self.dim)
+        return self.o.forward(gated, ctx)
+
+
+@dataclasses.dataclass(frozen=True)
+class MatrixMemoryNames:
+    q: str = "q"
+    k: str = "k"
+    v: str = "v"
+    gate: str = "g"
+    out: str = "o"
+    norm: str = "norm"
+    input_gate: str = "i"
+    forget_gate: str = "f"
+    bias_suffix: str = ".b"
+
+
+class MatrixMemory(Mixer):
+    """The matrix memory of xLSTM (mLSTM).  Per head, ``q = W_q h * dim^-1/2``, ``k``, ``v``; a log input gate
+    ``i = cap * tanh((W_i h + b_i) / cap)`` and a log forget gate ``f = logsigmoid(cap * tanh((W_f h + b_f) / cap))``.
+    With a running maximum ``m`` that starts at 0: ``m_t = max(f + m_(t-1), i)``, ``a = exp(f + m_(t-1) - m_t)``,
+    ``b = exp(i - m_t)``, ``S_t = a S_(t-1) + b k v^T``, ``n_t = a n_(t-1) + b k``,
+    ``o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + floor)``.  Each head's ``o`` is divided by its root mean square, the
+    heads side by side are multiplied by a weight per channel and by ``sigmoid(W_g h)``, then the output projection.
+
+    The gates' product leaves 32-bit numbers, and everything behind it (caps, logarithms, exponentials, maximum, state,
+    normaliser, read-out, norm) is 32-bit.  State per request: the matrices ``[heads, dim, vdim]``, behind them the
+    normalisers ``[heads, dim]`` and the maxima ``[heads]``; zeros before a sequence's first token."""
+    graph_safe = True
+
+    def __init__(self, width: int, heads: int, dim: int, value_dim: int, gate_cap: float, norm_eps: float, floor: float = 1e-6,
+                 names: MatrixMemoryNames = MatrixMemoryNames()):
+        self.width, self.heads, self.dim, self.value_dim = width, heads, dim, value_dim
+        self.gate_cap, self.norm_eps, self.floor, self.names = float(gate_cap), float(norm_eps), float(floor), names
+        self.q_scale = float(dim) ** -0.5
+        keys, values = heads * dim, heads * value_dim
+        # queries, keys, values and output gates read the same input: one product; the two gates of the recurrence are a
+        # product of their own, whose sums stay in 32-bit
+        self.proj = Linear(width, (names.q, names.k, names.v, names.gate), (keys, keys, values, values), bare_names=True)
+        self.gates = Linear(width, (names.input_gate, names.forget_gate), (heads, heads), bias=True, out_float32=True, bare_names=True,
+                            bias_suffix=names.bias_suffix)
+        self.o = Linear(values, (names.out,), (width,), bare_names=True)
+        self.norm_weight = None
+        self.matrix_size, self.normaliser_size = heads * dim * value_dim, heads * dim
+
+    def cache_spec(self):
+        return StateSpec((self.matrix_size + self.normaliser_size + self.heads,), "float32")
+
+    def param_specs(self):
+        specs = {**self.proj.param_specs(), **self.gates.param_specs(), **self.o.param_specs()}
+        specs[self.names.norm] = ParamSpec((self.heads * self.value_dim,), VECTOR, "norm")
+        return specs
+
+    def assign(self, name, tensor):
+        if name == self.names.norm:
+            self.norm_weight = tensor
+        elif self.gates.owns(name):
+            self.gates.assign(name, tensor)
+        elif self.o.owns(name):
+            self.o.assign(name, tensor)
+        elif self.proj.owns(name):
+            self.proj.assign(name, tensor)
+        else:
+            raise KeyError(name)
+
+    def finalize(self):
+        for part in (self.proj, self.gates, self.o):
+            part.finalize()
+
+    def mixing_flops(self, new_tokens: int, context: int) -> float:
+        """Per token, head and state element: the decay, the outer product's sum and the read-out."""
+        return 6.0 * new_tokens * self.heads * self.dim * self.value_dim
+
+    def forward(self, x, ctx, cache):
+        ops = ctx.ops
+        n = x.shape[0]
+        keys, values = self.heads * self.dim, self.heads * self.value_dim
+        proj = self.proj.forward(x, ctx)
+        q, k = proj[:, :keys], proj[:, keys:2 * keys]
+        v, gate = proj[:, 2 * keys:2 * keys + values], proj[:, 2 * keys + values:]
+        gates = self.gates.forward(x, ctx)                                           # float32 [T, input gates | forget gates]
+        # the memory leaves the read-outs' numerators and, per token and head, what stands below them (n . q and exp(-m));
+        # the division is the first thing the kernel of the heads' norm does
+        mixed = ctx.empty((n, values), dtype=torch.float32)
+        below = ctx.empty((n, self.heads, 2), dtype=torch.float32)
+        coefficients = ctx.empty((n, self.heads, 2), dtype=torch.float32)
+        ops.matrix_memory(q, k, v, gates, self.gate_cap, self.q_scale, cache.state, ctx.state_slots, ctx.row_start, ctx.row_len, ctx.row_ctx,
+                          mixed, below, coefficients, self.heads, self.dim, self.value_dim)
+        gated = ctx.empty((n, values))
+        ops.heads_norm_gate(mixed, self.norm_weight, True, self.norm_eps, gate, gated, self.heads, self.value_dim, gate_activation="sigmoid",
+                            below=below, floor=self.floor)
         return self.o.forward(gated, ctx)

@@ -16,14 +16,22 @@ from .base import PositionEncoding
 
 
 class RotaryPosition(PositionEncoding):
-    def __init__(self, rotary_dim: int, theta: float):
+    """``rotary_dim`` may be smaller than the head it is applied to: dimension ``i`` then turns with ``i + rotary_dim / 2``
+    and the dimensions behind ``rotary_dim`` pass unchanged (a mixer says whether its kernels do that).  ``precise``: the
+    frequencies are formed in 64-bit and rounded to 32-bit once, instead of with the 32-bit expression above."""
+    pairing = "halves"
+
+    def __init__(self, rotary_dim: int, theta: float, precise: bool = False):
         if rotary_dim % 2:
             raise ValueError(f"rotary_dim must be even: {rotary_dim}")
         self.rotary_dim = rotary_dim
         self.theta = float(theta)
+        self.precise = bool(precise)
         self._tables = {}
 
     def inverse_frequencies(self) -> torch.Tensor:
+        if self.precise:
+            return torch.tensor([self.theta ** (-2.0 * i / self.rotary_dim) for i in range(self.rotary_dim // 2)], dtype=torch.float32)
         indices = torch.arange(0, self.rotary_dim, 2, dtype=torch.long)
         return 1.0 / (self.theta ** (indices.to(torch.float32) / self.rotary_dim))
 

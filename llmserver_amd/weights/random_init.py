@@ -4,7 +4,7 @@ The reference's loader has no such mode; its tests seed a generator and draw eve
 from a normal distribution (tests/test_paged_decode.py:273-277).  Here each
 tensor is drawn from a generator seeded by (seed, tensor name), so the values do not depend on
 the order of tensors: matrices ``N(0, std)``, norm weights ``1 + N(0, norm_noise)``, biases
-``N(0, bias_std)``.
+``N(0, bias_std)``, small square mixing matrices ``I + N(0, bias_std)``.
 """
 from __future__ import annotations
 
@@ -48,6 +48,8 @@ def random_tensor(name: str, spec: ParamSpec, init: RandomInit, device="cpu") ->
         return init.bias_std * values
     if spec.init == "zeros":
         return torch.zeros_like(values)
+    if spec.init == "identity":          # a square matrix around the identity
+        return torch.eye(spec.shape[0], device=device, dtype=torch.float32) + init.bias_std * values
     return init.std * values
 
 

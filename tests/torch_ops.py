@@ -200,8 +200,22 @@ class TorchOps(KernelNamespace):
     def embedding_norm(self, table, token_ids, weight, eps, out):
         out.copy_(self._rms(table[token_ids.long()].float(), eps) * weight)
 
-    def embedding_wide(self, table, token_ids, out):
-        out.copy_(table[token_ids.long()].float())
+    def embedding_wide(self, table, token_ids, out, scale=1.0):
+        out.copy_(table[token_ids.long()].float() * scale)        # (several streams: the rows once for each)
+
+    def streams_read(self, streams, read, weight, eps, out, rows=None):
+        picked = streams if rows is None else streams[:, rows.long()]
+        out.copy_((self._rms((picked * read[:, None, None]).sum(dim=0), eps) * weight).to(out.dtype))
+
+    def streams_update(self, streams, y, mix, write, next_read=None, next_weight=None, next_eps=0.0, normed=None):
+        new = torch.einsum("st,snw->tnw", mix, streams) + write[:, None, None] * y.float()[None]
+        streams.copy_(new)
+        if next_read is not None:
+            self.streams_read(streams, next_read, next_weight, next_eps, normed)
+
+    def activation_(self, x, activation):
+        z = x.float()
+        x.copy_((torch.relu(z) ** 2 if activation == "relu2" else self._activated(z, activation)).to(x.dtype))
 
     def norm_add_norm(self, x, y, weight, eps, out, next_weight=None, next_eps=0.0, normed=None, y2=None, scales=None):
         update = y.float() if y2 is None else scales[0] * y.float() + scales[1] * y2.float()
@@ -263,7 +277,7 @@ class TorchOps(KernelNamespace):
 
     # -- general preparation of queries, keys and values -------------------------------------------------
     def qkv_prepare(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
-                    n_q, n_kv, dim, value_dim, out_q, write_cache=True):
+                    n_q, n_kv, dim, value_dim, out_q, write_cache=True, pairing="neighbours"):
         n, width = qkv.shape[0], keys.shape[-1]
         q = qkv[:, :n_q * dim].float().view(n, n_q, dim)
         k = qkv[:, n_q * dim:(n_q + n_kv) * dim].float().view(n, n_kv, dim)
@@ -275,6 +289,9 @@ class TorchOps(KernelNamespace):
             cos, sin = cos_sin[:, None, :pairs], cos_sin[:, None, pairs:]
 
             def turned(x):
+                if pairing == "halves":
+                    a, b = x[..., :pairs], x[..., pairs:2 * pairs]
+                    return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., 2 * pairs:]], dim=-1)
                 a, b = x[..., 0:2 * pairs:2], x[..., 1:2 * pairs:2]
                 return torch.cat([torch.stack([a * cos - b * sin, b * cos + a * sin], dim=-1).flatten(-2), x[..., 2 * pairs:]], dim=-1)
             q, k = turned(q), turned(k)
@@ -351,12 +368,46 @@ class TorchOps(KernelNamespace):
                     matrix = d * matrix + kv
             state[slot, offset:offset + size] = matrix.reshape(-1)
 
-    def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim):
+    def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim, gate_activation="silu", below=None, floor=0.0):
         n = x.shape[0]
-        normed = self._rms(x.float().view(n, heads, value_dim), eps)
+        rows = x.float().view(n, heads, value_dim)
+        if below is not None:
+            rows = rows / (torch.maximum(below[..., 0].abs(), below[..., 1]) + floor)[..., None]
+        normed = self._rms(rows, eps)
         normed = normed * (weight.view(heads, value_dim) if weight_per_channel else weight)
-        g = gate.float().view(n, heads, value_dim)
-        out.copy_((normed * g * torch.sigmoid(g)).reshape(n, heads * value_dim).to(out.dtype))
+        g = gate.float().reshape(n, heads, value_dim)
+        g = torch.sigmoid(g) if gate_activation == "sigmoid" else g * torch.sigmoid(g)
+        out.copy_((normed * g).reshape(n, heads * value_dim).to(out.dtype))
+
+    def matrix_memory(self, q, k, v, gates, cap, q_scale, state, state_slots, row_start, row_len, row_ctx, out, below, coefficients,
+                      heads, dim, value_dim):
+        matrix_size, normaliser_size = heads * dim * value_dim, heads * dim
+        log_in = cap * torch.tanh(gates[:, :heads].float() / cap)
+        log_forget = torch.nn.functional.logsigmoid(cap * torch.tanh(gates[:, heads:].float() / cap))
+        for row in range(len(row_len)):
+            start, count, end = int(row_start[row]), int(row_len[row]), int(row_ctx[row])
+            if count <= 0:
+                continue
+            slot = int(state_slots[row])
+            kept = state[slot].clone()
+            if end - count == 0:
+                kept.zero_()
+            matrix = kept[:matrix_size].view(heads, dim, value_dim)
+            normaliser = kept[matrix_size:matrix_size + normaliser_size].view(heads, dim)
+            top = kept[matrix_size + normaliser_size:matrix_size + normaliser_size + heads]
+            for t in range(start, start + count):
+                qt, kt = q[t].float().view(heads, dim) * q_scale, k[t].float().view(heads, dim)
+                new_top = torch.maximum(log_forget[t] + top, log_in[t])
+                keep, take = torch.exp(log_forget[t] + top - new_top), torch.exp(log_in[t] - new_top)
+                matrix = keep[:, None, None] * matrix + take[:, None, None] * kt[:, :, None] * v[t].float().view(heads, value_dim)[:, None, :]
+                normaliser = keep[:, None] * normaliser + take[:, None] * kt
+                top = new_top
+                coefficients[t, :, 0], coefficients[t, :, 1] = keep, take
+                below[t, :, 0], below[t, :, 1] = (normaliser * qt).sum(dim=-1), torch.exp(-top)
+                out[t] = torch.einsum("hdv,hd->hv", matrix, qt).reshape(-1)
+            state[slot, :matrix_size] = matrix.reshape(-1)
+            state[slot, matrix_size:matrix_size + normaliser_size] = normaliser.reshape(-1)
+            state[slot, matrix_size + normaliser_size:matrix_size + normaliser_size + heads] = top
 
     def scaled_sum(self, x, x_scale, y, y_scale, out):
         out.copy_((x_scale * x.float() + y_scale * y.float()).to(out.dtype))
@@ -398,12 +449,16 @@ class TorchOps(KernelNamespace):
         keys[pages, 0, slots, :] = row.to(keys.dtype)
         values[pages, 0, :, slots] = row.to(values.dtype)
 
-    def gate_heads(self, y, proj, gate_column, out, mixed=None, up_values=None):
+    def gate_heads(self, y, proj, gate_column, out, mixed=None, up_values=None, per_channel=False):
         if y is None:
             heads, rank, _ = up_values.shape
             rows = mixed.float().view(mixed.shape[0], heads, -1)[:, :, :rank]
             y = torch.einsum("thr,hrv->htv", rows, up_values.float())
         heads, n, v = y.shape
+        if per_channel and gate_column >= 0:
+            gate = torch.sigmoid(proj[:, gate_column:gate_column + heads * v].float()).view(n, heads, v)
+            out.copy_((y.float().transpose(0, 1) * gate).reshape(n, heads * v).to(out.dtype))
+            return
         gate = torch.sigmoid(proj[:, gate_column:gate_column + heads].float()) if gate_column >= 0 else torch.ones(n, heads, device=y.device)
         out.copy_((y.float().transpose(0, 1) * gate[..., None]).reshape(n, heads * v).to(out.dtype))
 
