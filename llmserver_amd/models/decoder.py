@@ -47,6 +47,7 @@ class DecoderModel:
         self.embed_name, self.layers_name, self.norm_name = names
         self.layer_name = layer_name if layer_name is not None else (lambda index: f"{self.layers_name}.{index}")
         self._owners = None
+        self.after_call = None      # for whoever looks inside a step: called as (index in the order, residual, pending update) behind every call
         self.device = None
         self.dtype = None
         self._check_order()
@@ -135,6 +136,8 @@ class DecoderModel:
                 resid, delta = block.forward(resid, delta, ctx, caches.view(call), following=following)
             else:
                 resid, delta = block.forward(resid, delta, ctx, caches.view(call))
+            if self.after_call is not None:
+                self.after_call(index, delta.resid if isinstance(delta, StreamUpdate) else resid, delta)
         if isinstance(delta, StreamUpdate):
             resid, delta = delta.resid, None
         if ctx.n_out == 0:

@@ -99,12 +99,17 @@ def test_pools_that_let_a_context_outgrow_the_kernels_page_lookup_are_refused():
 
 
 def test_parts_refuse_what_their_kernels_do_not_compute_when_they_are_made():
-    """A position encoding that rotates a part of the head, or an activation that the kernels do not compute, is refused
-    with the reason by the part's constructor, not by a shape check at the first step."""
-    from llmserver_amd.parts import GatedMLP, GQAttention, NoPosition, RotaryPosition
-    with pytest.raises(ValueError, match="rotates 16 of a head's 32 dimensions"):
-        GQAttention(64, 4, 2, 32, RotaryPosition(16, 1e4))
+    """A position encoding that rotates more dimensions than a head has, or an activation that the kernels do not compute,
+    is refused with the reason by the part's constructor, not by a shape check at the first step.  (A rotation of a part
+    of the head goes the general way of preparing queries and keys.)"""
+    from llmserver_amd.parts import GatedMLP, GQAttention, NoPosition, PlainMLP, RotaryPosition
+    with pytest.raises(ValueError, match="rotates 48 dimensions, a head has 32"):
+        GQAttention(64, 4, 2, 32, RotaryPosition(48, 1e4))
+    assert GQAttention(64, 4, 2, 32, RotaryPosition(16, 1e4)).general
+    assert not GQAttention(64, 4, 2, 32, RotaryPosition(32, 1e4)).general
     assert GQAttention(64, 4, 2, 32, RotaryPosition(32, 1e4)).position.rotary_dim == 32
+    with pytest.raises(ValueError, match="Unsupported activation 'relu'"):
+        PlainMLP(64, 128, "relu")
     assert GQAttention(64, 4, 2, 32, NoPosition()).position.rotary_dim is None
     with pytest.raises(ValueError, match="Unsupported activation 'gelu'"):
         GatedMLP(64, 128, "gelu")
