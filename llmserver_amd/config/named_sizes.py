@@ -78,6 +78,27 @@ NAMED_SIZES.update({
 })
 
 
+def _kerudra(width, layers, heads, kv_heads, dim, window, rot_dim, kv_rank, memory_heads, memory_dim, memory_vdim, ff, streams=2, vocab=32768):
+    memory = ("mlstm", {"heads": memory_heads, "dim": memory_dim, "vdim": memory_vdim, "gate_cap": 15.0})
+    latent = ("latent_attention", {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": dim, "kv_rank": kv_rank, "scale": (dim + rot_dim) ** -0.5,
+                                   "rot": {"base": 10000.0, "dims": rot_dim}, "mask": {"size": window}})
+    attention = ("attention", {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "rot": {"base": 10000.0, "dims": dim}})
+    four = [memory, latent, attention, memory]
+    return {"architecture": "Kerudra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "streams": streams, "residual_mult": 0.5,
+            "embedding": {"scale": 1.0}, "logit_scale": 1.0,
+            "layers": [{"type": kind, "mixer": dict(mixer), "mlp": {"kind": "dense", "ff": ff}} for kind, mixer in (four * (-(-layers // 4)))[:layers]]}
+
+
+# Kerudra at the widths of the sizes above, two residual streams: of every four layers two are matrix memories of 8 (16)
+# heads with keys of 128 and values of 256 (a state of 1 MB a layer and request), one is latent attention of the Zepolix
+# sizes' shape under a window of 1,024 keys and a gate per channel, one is attention of 16 (32) heads of 128 over 8 key/value
+# heads whose values are its keys; plain feed-forwards as wide as the dense decoders' gated ones beside them.
+NAMED_SIZES.update({
+    "kerudra-2k": _kerudra(2048, 8, 16, 8, 128, 1024, 64, 192, 8, 128, 256, 6 * 1408),
+    "kerudra-4k": _kerudra(4096, 8, 32, 8, 128, 1024, 64, 192, 16, 128, 256, 4 * 2048),
+})
+
+
 def named_size(name: str) -> dict:
     """The entry's keys, a copy the caller may change (fewer layers, say)."""
     try:
