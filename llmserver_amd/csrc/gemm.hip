@@ -45,7 +45,18 @@ struct Fusion {
     float* square_sums_out;              // [M, P], P as lsa_gemm_skinny_parts tells
     // Bias (null: none), added to the float32 sum before its one rounding; plain results only.
     const float* bias;                   // [N]
+    // What the sum (with its bias) goes through before its one rounding; plain results only.
+    // 0: nothing, 1: z sigmoid(z), 2: the tanh form of GELU, 3: max(z, 0)^2.
+    int activation;
 };
+
+__device__ inline float plain_result(const Fusion& f, float z, int n) {
+    if (f.bias) z += f.bias[n];
+    if (f.activation == 1) return z / (1.f + expf(-z));
+    if (f.activation == 2) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    if (f.activation == 3) { const float r = fmaxf(z, 0.f); return r * r; }
+    return z;
+}
 
 // The partial sums of wavefront `wave`'s row are loaded behind the last operands of the product
 // (they come from cache and are there by the time those have arrived) and while few registers
@@ -223,7 +234,7 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
             if (j == 0 && m < M) fusion.square_sums_out[(size_t)m * gridDim.x + blockIdx.x] = sq;
             continue;
         }
-        if (m < M && j < R && n < N) y[(size_t)m * N + n] = (OutT)(fusion.bias ? total + fusion.bias[n] : total);
+        if (m < M && j < R && n < N) y[(size_t)m * N + n] = (OutT)plain_result(fusion, total, n);
     }
 }
 
@@ -343,7 +354,7 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_wide_kernel(const
         if (!tile && j == 0 && m < M) fusion.square_sums_out[(size_t)m * gridDim.x + blockIdx.x] = sq + second_tile_sums[m];
         return;
     }
-    if (m < M && own && n < N) y[(size_t)m * N + n] = (OutT)(fusion.bias ? total + fusion.bias[n] : total);
+    if (m < M && own && n < N) y[(size_t)m * N + n] = (OutT)plain_result(fusion, total, n);
 }
 
 // The chunk size in 4..8 that wastes the fewest loads past the end of a wavefront's share of K.
@@ -681,14 +692,14 @@ static bool fusion_fits(int M, const float* square_sums, int n_parts, const void
 
 // out_float32: 0 writes bfloat16, 1 writes float32.  rows: rows of W per workgroup, 1 to 32 (more than 16
 // only for M <= 16), or 0 to let the size decide.  square_sums [M, n_parts] (or null) asks for the row scale
-// rsqrt(sum / K + eps), M <= 16.  bias [N] (or null) is added to the sums before they are rounded.  Refuses
-// (returns -1) what it cannot take.
+// rsqrt(sum / K + eps), M <= 16.  bias [N] (or null) is added to the sums before they are rounded, and the sums go through
+// `activation` (Fusion's codes; 0: none) before that rounding.  Refuses (returns -1) what it cannot take.
 LSA_EXPORT int lsa_gemm_skinny(int out_float32, const void* x, const void* w, void* y, int M, int N, int K, int rows,
-                               const float* square_sums, int n_parts, float eps, const float* bias, hipStream_t stream) {
+                               const float* square_sums, int n_parts, float eps, const float* bias, int activation, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 64 || K % 8 != 0 || K < 8 || rows < 0 || rows > 32 || (rows > 16 && M > 16)) return -1;
+    if (M > 64 || K % 8 != 0 || K < 8 || rows < 0 || rows > 32 || (rows > 16 && M > 16) || activation < 0 || activation > 3) return -1;
     if (!fusion_fits(M, square_sums, n_parts, nullptr)) return -1;
-    const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr, bias};
+    const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr, bias, activation};
     rows = choose_rows(M, N, false, rows);
     return out_float32 ? launch<float, false>((const bf16_t*)x, (const bf16_t*)w, (float*)y, M, N, K, rows, fusion, stream)
                        : launch<bf16_t, false>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, rows, fusion, stream);
@@ -727,7 +738,7 @@ LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* h
     if (M <= 0 || I <= 0) return 0;
     if (M > 16 || K % 8 != 0 || K < 8 || I % 8 != 0 || rows < -1 || rows > 16) return -1;
     if (!fusion_fits(M, square_sums, n_parts, nullptr)) return -1;
-    const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     return launch<bf16_t, true>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)hidden, M, 2 * I, K, choose_rows(M, 2 * I, true, rows),
                                 fusion, stream);
 }

@@ -201,82 +201,108 @@ __global__ __launch_bounds__(256) void embedding_wide_kernel(const T* __restrict
 constexpr int MOST_STREAMS = 8;
 constexpr int STREAM_CACHE = 8;           // elements of a row a thread keeps between the two passes (rows of up to 2,048 are read once)
 
+// The kernels below take the number of streams as a template parameter: the small per-stream arrays then live in registers
+// (indexed by a run-time count they would go to scratch memory, and a row of one token would wait for that).
 // out[i] = rmsnorm(sum_s read[s] * x[s][rows[i]]) * weight (rows == nullptr: every row).
-template <typename O>
-__global__ __launch_bounds__(256) void streams_read_kernel(const float* __restrict__ x, size_t stream_stride, int streams,
+template <typename O, int S>
+__global__ __launch_bounds__(256) void streams_read_kernel(const float* __restrict__ x, size_t stream_stride,
                                                            const float* __restrict__ read, const int* __restrict__ rows,
                                                            const float* __restrict__ weight, float eps, O* __restrict__ out, int width) {
     __shared__ float scratch[16];
     const float* row = x + (size_t)(rows ? rows[blockIdx.x] : blockIdx.x) * width;
-    float r[MOST_STREAMS];
-    for (int s = 0; s < MOST_STREAMS; ++s) r[s] = s < streams ? read[s] : 0.f;
+    float r[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) r[s] = read[s];
     auto summed = [&](int i) {
         float u = 0.f;
-        for (int s = 0; s < streams; ++s) u += r[s] * row[(size_t)s * stream_stride + i];
+#pragma unroll
+        for (int s = 0; s < S; ++s) u += r[s] * row[(size_t)s * stream_stride + i];
         return u;
     };
     float kept[STREAM_CACHE];
     float sq = 0.f;
-    int k = 0;
-    for (int i = threadIdx.x; i < width; i += blockDim.x, ++k) {
+#pragma unroll
+    for (int k = 0; k < STREAM_CACHE; ++k) {
+        const int i = threadIdx.x + k * 256;
+        kept[k] = i < width ? summed(i) : 0.f;
+        sq += kept[k] * kept[k];
+    }
+    for (int i = threadIdx.x + STREAM_CACHE * 256; i < width; i += 256) {
         const float u = summed(i);
-        if (k < STREAM_CACHE) kept[k] = u;
         sq += u * u;
     }
     const float inv = rsqrtf(block_sum(sq, scratch) / (float)width + eps);
     O* o = out + (size_t)blockIdx.x * width;
-    k = 0;
-    for (int i = threadIdx.x; i < width; i += blockDim.x, ++k) o[i] = (O)((k < STREAM_CACHE ? kept[k] : summed(i)) * inv * weight[i]);
+#pragma unroll
+    for (int k = 0; k < STREAM_CACHE; ++k) {
+        const int i = threadIdx.x + k * 256;
+        if (i < width) o[i] = (O)(kept[k] * inv * weight[i]);
+    }
+    for (int i = threadIdx.x + STREAM_CACHE * 256; i < width; i += 256) o[i] = (O)(summed(i) * inv * weight[i]);
 }
 
 // All streams at once from the old ones, where they lie: x[t] <- sum_s mix[s][t] * x[s] + write[t] * y, and, where next_read
 // is given, normed = rmsnorm(sum_t next_read[t] * x[t]) * next_weight: what the next sublayer reads, in the same pass (the
 // row of sums stays in registers between the two passes; wider rows are formed again from the streams just written, by the
 // thread that wrote them).  One workgroup a token row.
-template <typename Y, typename R>
-__global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__ x, size_t stream_stride, int streams, const Y* __restrict__ y,
+template <typename Y, typename R, int S>
+__global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__ x, size_t stream_stride, const Y* __restrict__ y,
                                                              const float* __restrict__ mix, const float* __restrict__ write,
                                                              const float* __restrict__ next_read, const float* __restrict__ next_weight,
                                                              float next_eps, R* __restrict__ normed, int width) {
     __shared__ float scratch[16];
-    __shared__ float s_mix[MOST_STREAMS * MOST_STREAMS], s_write[MOST_STREAMS], s_read[MOST_STREAMS];
-    if (threadIdx.x < streams * streams) s_mix[threadIdx.x] = mix[threadIdx.x];
-    if (threadIdx.x < streams) {
-        s_write[threadIdx.x] = write[threadIdx.x];
-        s_read[threadIdx.x] = next_read ? next_read[threadIdx.x] : 0.f;
+    float m[S][S], w[S], r[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+#pragma unroll
+        for (int t = 0; t < S; ++t) m[s][t] = mix[s * S + t];
+        w[s] = write[s];
+        r[s] = next_read ? next_read[s] : 0.f;
     }
-    __syncthreads();
     float* row = x + (size_t)blockIdx.x * width;
     const Y* yr = y + (size_t)blockIdx.x * width;
-    float kept[STREAM_CACHE];
-    float sq = 0.f;
-    int k = 0;
-    for (int i = threadIdx.x; i < width; i += blockDim.x, ++k) {
-        float old[MOST_STREAMS];
-        for (int s = 0; s < streams; ++s) old[s] = row[(size_t)s * stream_stride + i];
+    // one column of all streams: the new streams are written, what the next sublayer reads of them is returned
+    auto updated = [&](int i) {
+        float old[S];
+#pragma unroll
+        for (int s = 0; s < S; ++s) old[s] = row[(size_t)s * stream_stride + i];
         const float update = (float)yr[i];
         float u = 0.f;
-        for (int t = 0; t < streams; ++t) {
+#pragma unroll
+        for (int t = 0; t < S; ++t) {
             float fresh = 0.f;
-            for (int s = 0; s < streams; ++s) fresh += s_mix[s * streams + t] * old[s];
-            fresh += s_write[t] * update;
+#pragma unroll
+            for (int s = 0; s < S; ++s) fresh += m[s][t] * old[s];
+            fresh += w[t] * update;
             row[(size_t)t * stream_stride + i] = fresh;
-            u += s_read[t] * fresh;
+            u += r[t] * fresh;
         }
-        if (k < STREAM_CACHE) kept[k] = u;
+        return u;
+    };
+    float kept[STREAM_CACHE];
+    float sq = 0.f;
+#pragma unroll
+    for (int k = 0; k < STREAM_CACHE; ++k) {
+        const int i = threadIdx.x + k * 256;
+        kept[k] = i < width ? updated(i) : 0.f;
+        sq += kept[k] * kept[k];
+    }
+    for (int i = threadIdx.x + STREAM_CACHE * 256; i < width; i += 256) {
+        const float u = updated(i);
         sq += u * u;
     }
     if (!next_read) return;                              // (the whole workgroup)
     const float inv = rsqrtf(block_sum(sq, scratch) / (float)width + next_eps);
     R* o = normed + (size_t)blockIdx.x * width;
-    k = 0;
-    for (int i = threadIdx.x; i < width; i += blockDim.x, ++k) {
-        float u;
-        if (k < STREAM_CACHE) u = kept[k];
-        else {
-            u = 0.f;
-            for (int t = 0; t < streams; ++t) u += s_read[t] * row[(size_t)t * stream_stride + i];
-        }
+#pragma unroll
+    for (int k = 0; k < STREAM_CACHE; ++k) {
+        const int i = threadIdx.x + k * 256;
+        if (i < width) o[i] = (R)(kept[k] * inv * next_weight[i]);
+    }
+    for (int i = threadIdx.x + STREAM_CACHE * 256; i < width; i += 256) {
+        float u = 0.f;
+#pragma unroll
+        for (int t = 0; t < S; ++t) u += r[t] * row[(size_t)t * stream_stride + i];
         o[i] = (R)(u * inv * next_weight[i]);
     }
 }
@@ -373,8 +399,13 @@ LSA_EXPORT int lsa_streams_read(const float* x, int streams, int n_tokens, const
     if (n_out <= 0) return 0;
     if (streams < 1 || streams > MOST_STREAMS) return -1;
     const size_t stream_stride = (size_t)n_tokens * width;
-    if (out_code) streams_read_kernel<bf16_t><<<n_out, 256, 0, stream>>>(x, stream_stride, streams, read, rows, weight, eps, (bf16_t*)out, width);
-    else streams_read_kernel<float><<<n_out, 256, 0, stream>>>(x, stream_stride, streams, read, rows, weight, eps, (float*)out, width);
+#define LSA_LAUNCH(O, S) streams_read_kernel<O, S><<<n_out, 256, 0, stream>>>(x, stream_stride, read, rows, weight, eps, (O*)out, width)
+#define LSA_BY_STREAMS(O) switch (streams) { case 1: LSA_LAUNCH(O, 1); break; case 2: LSA_LAUNCH(O, 2); break; case 3: LSA_LAUNCH(O, 3); break; \
+        case 4: LSA_LAUNCH(O, 4); break; case 5: LSA_LAUNCH(O, 5); break; case 6: LSA_LAUNCH(O, 6); break; case 7: LSA_LAUNCH(O, 7); break; \
+        default: LSA_LAUNCH(O, 8); }
+    if (out_code) LSA_BY_STREAMS(bf16_t) else LSA_BY_STREAMS(float)
+#undef LSA_BY_STREAMS
+#undef LSA_LAUNCH
     LSA_LAUNCH_CHECK();
 }
 
@@ -384,13 +415,17 @@ LSA_EXPORT int lsa_streams_update(float* x, int streams, int n_tokens, const voi
     if (n_tokens <= 0) return 0;
     if (streams < 1 || streams > MOST_STREAMS || (next_read != nullptr && (normed == nullptr || next_weight == nullptr))) return -1;
     const size_t stream_stride = (size_t)n_tokens * width;
-#define LSA_LAUNCH(Y, R) streams_update_kernel<Y, R><<<n_tokens, 256, 0, stream>>>(x, stream_stride, streams, (const Y*)y, mix, write, next_read, \
-                                                                                  next_weight, next_eps, (R*)normed, width)
-    if (y_code && normed_code) LSA_LAUNCH(bf16_t, bf16_t);
-    else if (y_code) LSA_LAUNCH(bf16_t, float);
-    else if (normed_code) LSA_LAUNCH(float, bf16_t);
-    else LSA_LAUNCH(float, float);
+#define LSA_LAUNCH_S(Y, R, S) streams_update_kernel<Y, R, S><<<n_tokens, 256, 0, stream>>>(x, stream_stride, (const Y*)y, mix, write, next_read, \
+                                                                                          next_weight, next_eps, (R*)normed, width)
+#define LSA_LAUNCH(Y, R) switch (streams) { case 1: LSA_LAUNCH_S(Y, R, 1); break; case 2: LSA_LAUNCH_S(Y, R, 2); break; case 3: LSA_LAUNCH_S(Y, R, 3); break; \
+        case 4: LSA_LAUNCH_S(Y, R, 4); break; case 5: LSA_LAUNCH_S(Y, R, 5); break; case 6: LSA_LAUNCH_S(Y, R, 6); break; \
+        case 7: LSA_LAUNCH_S(Y, R, 7); break; default: LSA_LAUNCH_S(Y, R, 8); }
+    if (y_code && normed_code) LSA_LAUNCH(bf16_t, bf16_t)
+    else if (y_code) LSA_LAUNCH(bf16_t, float)
+    else if (normed_code) LSA_LAUNCH(float, bf16_t)
+    else LSA_LAUNCH(float, float)
 #undef LSA_LAUNCH
+#undef LSA_LAUNCH_S
     LSA_LAUNCH_CHECK();
 }
 

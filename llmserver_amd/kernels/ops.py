@@ -373,14 +373,26 @@ class HipOps(KernelNamespace):
             self.add_bias_(y, bias)
         return y
 
-    def linear_few_rows(self, x, weight, out=None, out_float32=False, rows_per_workgroup=0, row_scale=None, bias=None):
+    def linear_activated(self, x, weight, activation):
+        """``act(x @ weight^T)``, the activation computed on the 32-bit sums where the few-row kernel forms them (one
+        rounding), behind the library's product otherwise."""
+        if self._few_rows(x, weight) and not self.library_is_faster("plain", x, weight, False, False):
+            return self.linear_few_rows(x, weight, activation=activation)
+        y = self.linear(x, weight)
+        self.activation_(y, activation)
+        return y
+
+    def linear_few_rows(self, x, weight, out=None, out_float32=False, rows_per_workgroup=0, row_scale=None, bias=None, activation=None):
         """The weight-streaming product, or None if this is no case for it.
 
         ``row_scale = (square_sums [T, P], eps)``: ``x`` is a residual stream already multiplied by a norm's
         weights, ``square_sums`` are partial sums of the stream's squares, and the result rows are divided by the
         stream's root mean square, so that the result is the product of the normalised stream (up to 16 rows).
-        ``bias [out]`` (float32) is added before the result is rounded."""
+        ``bias [out]`` (float32) is added before the result is rounded; ``activation`` (one of ``PLAIN_ACTIVATIONS``) is
+        what the sums go through before that rounding."""
         rows, width = x.shape
+        if activation is not None and activation not in self.PLAIN_ACTIVATIONS:
+            raise ValueError(f"the product's epilogue computes {', '.join(self.PLAIN_ACTIVATIONS)}; {activation!r} is not built")
         if x.shape[1] != weight.shape[1] or not self._few_rows(x, weight) or not self._row_scale_fits(row_scale, rows) \
                 or (rows_per_workgroup > 16 and rows > 16):
             return None
@@ -394,7 +406,7 @@ class HipOps(KernelNamespace):
             _check(bias, "bias", torch.float32, (weight.shape[0],))
         _launched(self._gemm.lsa_gemm_skinny(1 if out_float32 else 0, _ptr(x), _ptr(weight), _ptr(out), rows, weight.shape[0], width,
                                              int(rows_per_workgroup), sums, parts, eps, _ptr(bias) if bias is not None else None,
-                                             _stream()), "gemm_skinny")
+                                             0 if activation is None else 1 + self.PLAIN_ACTIVATIONS.index(activation), _stream()), "gemm_skinny")
         return out
 
     SPLIT_ROWS = 128        # most rows the product that leaves partial sums takes (it starts above the few-row kernels')

@@ -129,6 +129,11 @@ class KernelNamespace:
         """``x = act(x)`` where it lies, in 32-bit, rounded once: ``"relu2"`` (``max(x, 0)^2``), ``"gelu_tanh"``, ``"silu"``."""
         raise NotImplementedError
 
+    def linear_activated(self, x, weight, activation):
+        """``act(x @ weight^T)`` in ``x``'s type, ``act`` as in :meth:`activation_`, computed on the product's 32-bit sums
+        where the kernel that forms them can (one rounding), on the rounded product otherwise."""
+        raise NotImplementedError
+
     def scaled_sum(self, x, x_scale, y, y_scale, out):
         raise NotImplementedError
 

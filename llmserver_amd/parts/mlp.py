@@ -88,7 +88,8 @@ class GatedMLP(FeedForward):
 
 class PlainMLP(FeedForward):
     """``down(act(up(x)))`` without a gate.  ``activation``: ``"relu2"`` (``max(z, 0)^2``), ``"gelu_tanh"`` or ``"silu"``,
-    computed in 32-bit and stored over the up projection's result.  ``names``: the checkpoint names of the two matrices."""
+    computed in 32-bit: on the up projection's sums before their one rounding where the few-row kernel forms them, over the
+    library's rounded result otherwise.  ``names``: the checkpoint names of the two matrices."""
 
     ACTIVATIONS = ("relu2", "gelu_tanh", "silu")
 
@@ -117,6 +118,5 @@ class PlainMLP(FeedForward):
         self.down.finalize()
 
     def forward(self, x, ctx):
-        hidden = self.up.forward(x, ctx)
-        ctx.ops.activation_(hidden, self.activation)
+        hidden = ctx.ops.linear_activated(x, self.up.weight, self.activation)
         return self.down.forward(hidden, ctx)

@@ -516,7 +516,7 @@ def test_skinny_gemm(ops, rows, n, k):
     finally:
         ops.skinny_rows = saved
     with pytest.raises(RuntimeError):
-        ops._gemm_refusal_check = ops._gemm.lsa_gemm_skinny(0, x.data_ptr(), w.data_ptr(), got16.data_ptr(), 65, n, k, 0, None, 0, 0.0, None, None)
+        ops._gemm_refusal_check = ops._gemm.lsa_gemm_skinny(0, x.data_ptr(), w.data_ptr(), got16.data_ptr(), 65, n, k, 0, None, 0, 0.0, None, 0, None)
         if ops._gemm_refusal_check != 0:
             raise RuntimeError("refused")
 

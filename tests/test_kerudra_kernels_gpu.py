@@ -187,3 +187,15 @@ def test_queries_and_keys_turned_in_halves_and_values_left_as_projected(ops, dty
     close(q[t, 0, :dim], want, dtype, "a query by hand")
     slot = int(table[0, t // page])
     close(results[0][2][slot, 0, :dim, t % page], src[n_q + n_kv], dtype, "a value by hand")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [1, 5, 16, 40, 300])
+def test_a_product_with_its_activation_in_the_epilogue(ops, dtype, rows):
+    """Few rows: the few-row kernel applies the activation to its 32-bit sums; many rows: the library's product and the
+    activation kernel behind it."""
+    twin = TorchOps()
+    x = torch.randn(rows, 136, device="cuda").to(dtype)
+    weight = (0.2 * torch.randn(203, 136, device="cuda")).to(dtype)
+    for activation in ("relu2", "gelu_tanh", "silu"):
+        close(ops.linear_activated(x, weight, activation), twin.linear_activated(x, weight, activation), dtype, f"{activation} {rows}")

@@ -213,6 +213,10 @@ class TorchOps(KernelNamespace):
         if next_read is not None:
             self.streams_read(streams, next_read, next_weight, next_eps, normed)
 
+    def linear_activated(self, x, weight, activation):
+        z = x.float() @ weight.float().t()
+        return (torch.relu(z) ** 2 if activation == "relu2" else self._activated(z, activation)).to(x.dtype)
+
     def activation_(self, x, activation):
         z = x.float()
         x.copy_((torch.relu(z) ** 2 if activation == "relu2" else self._activated(z, activation)).to(x.dtype))
