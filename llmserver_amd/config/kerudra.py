@@ -20,6 +20,7 @@ from .zepolix import _number
 
 MIXERS = ("attention", "latent_attention", "mlstm")
 FEED_FORWARDS = ("dense",)
+MOST_STREAMS = 8            # what the stream kernels are built for (csrc/stream.hip)
 
 
 def _optional_mapping(where: str, raw: Mapping[str, Any], key: str) -> Optional[Mapping[str, Any]]:
@@ -217,6 +218,8 @@ class KerudraConfig(ModelConfig):
             raise ConfigError(f"norm.eps must be positive: {self.norm_eps}")
         if self.streams < 0:
             raise ConfigError(f"streams must not be negative: {self.streams}")
+        if self.streams > MOST_STREAMS:
+            raise UnsupportedModelError(f"Model type {self.MODEL_TYPE!r}: {self.streams} residual streams; the stream kernels take up to {MOST_STREAMS}")
         if self.loop is not None and not (0 <= self.loop.start <= self.loop.stop <= len(self.layers) and self.loop.times >= 1):
             raise ConfigError(f"loop: layers {self.loop.start} to {self.loop.stop - 1} of {len(self.layers)}, {self.loop.times} times")
         for index, layer in enumerate(self.layers):

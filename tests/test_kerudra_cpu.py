@@ -85,6 +85,10 @@ def test_the_configuration_reads_back_and_refuses_what_is_not_built():
     other["loop"]["stop"] = 9
     with pytest.raises(ConfigError, match="loop"):
         config_from_dict(other)
+    other = copy_of(KA)
+    other["streams"] = 9
+    with pytest.raises(UnsupportedModelError, match="streams"):
+        config_from_dict(other)
 
 
 def test_the_model_declares_the_checkpoints_tensors_and_its_caches():
