@@ -229,11 +229,14 @@ __global__ __launch_bounds__(64) void heads_norm_gate_kernel(const float* __rest
 // tokens in chunks of 64, a lane a token for the transcendental functions, one lane for the maximum's walk through the
 // chunk (two dependent instructions a token).  gates [T][2 heads] (inputs, then forgets), coef [T][heads][2] (keep, take),
 // below [T][heads][2] (its second number is written here), top[slot][head] the maximum between steps (0 at position 0).
+// run (or nullptr) [T][heads]: the sum of log keep from the first token of a token's chunk of 64 (counted from the row's
+// first token of this step) up to the token itself, in 64-bit: what the chunked form of the memory forms its weights from.
 __global__ __launch_bounds__(64) void memory_gates_kernel(const float* __restrict__ gates, float cap, float* state, long state_stride,
                                                           long top_offset, const int* __restrict__ slots, const int* __restrict__ row_start,
                                                           const int* __restrict__ row_len, const int* __restrict__ row_ctx,
-                                                          float* __restrict__ coef, float* __restrict__ below, int heads) {
-    __shared__ float s_in[64], s_forget[64], s_top[65];
+                                                          float* __restrict__ coef, float* __restrict__ below, int heads,
+                                                          double* __restrict__ run) {
+    __shared__ __align__(16) float s_in[64], s_forget[64], s_top[68];
     const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const int count = row_len[row];
     if (count <= 0) return;
@@ -257,17 +260,45 @@ __global__ __launch_bounds__(64) void memory_gates_kernel(const float* __restric
         if (lane == 0) {
             float m = top;
             s_top[0] = m;
-            for (int t = 0; t < n; ++t) {
-                m = fmaxf(s_forget[t] + m, s_in[t]);
-                s_top[t + 1] = m;
+            if (n == 64) {                                             // a whole chunk: all loads first, then the chain alone
+                float fs[64], is[64], ms[64];
+#pragma unroll
+                for (int t4 = 0; t4 < 16; ++t4) {
+                    const float4 f4 = reinterpret_cast<const float4*>(s_forget)[t4], i4 = reinterpret_cast<const float4*>(s_in)[t4];
+                    fs[4 * t4] = f4.x; fs[4 * t4 + 1] = f4.y; fs[4 * t4 + 2] = f4.z; fs[4 * t4 + 3] = f4.w;
+                    is[4 * t4] = i4.x; is[4 * t4 + 1] = i4.y; is[4 * t4 + 2] = i4.z; is[4 * t4 + 3] = i4.w;
+                }
+#pragma unroll
+                for (int t = 0; t < 64; ++t) {
+                    m = fmaxf(fs[t] + m, is[t]);
+                    ms[t] = m;
+                }
+#pragma unroll
+                for (int t = 0; t < 64; ++t) s_top[t + 1] = ms[t];
+            } else {
+                for (int t = 0; t < n; ++t) {
+                    m = fmaxf(s_forget[t] + m, s_in[t]);
+                    s_top[t + 1] = m;
+                }
             }
         }
         __syncthreads();
+        float log_keep = 0.f;
         if (lane < n) {
             const float before = s_top[lane], now = s_top[lane + 1];
-            coef[(token * heads + head) * 2] = expf((log_forget + before) - now);
+            log_keep = (log_forget + before) - now;
+            coef[(token * heads + head) * 2] = expf(log_keep);
             coef[(token * heads + head) * 2 + 1] = expf(log_in - now);
             below[(token * heads + head) * 2 + 1] = expf(-now);
+        }
+        if (run != nullptr) {                                          // the chunk's running sum of log keep, token by token
+            double total = (double)log_keep;
+#pragma unroll
+            for (int step = 1; step < 64; step <<= 1) {
+                const double other = __shfl_up(total, step, 64);
+                if (lane >= step) total += other;
+            }
+            if (lane < n) run[token * heads + head] = total;
         }
         top = s_top[n];
     }
@@ -395,6 +426,237 @@ __global__ __launch_bounds__(512) void matrix_memory_kernel(const T* __restrict_
         if ((is_value || is_normaliser) && channel0 + i < dim) mine[(size_t)i * channel_stride] = S[i];
 }
 
+// ---- the matrix memory in chunks -------------------------------------------------------------------------------------
+// A row's tokens of a step in chunks of 64, counted from the row's first token of the step.  With L_t the sum of log keep
+// from the chunk's first token to t, the state behind token t is e^(L_t) S_0 + sum_(j <= t) e^(L_t - L_j) take_j k_j v_j^T
+// (S_0 the state in front of the chunk), and every weight is at most 1.  So (1) every chunk's own sum
+// U = sum_j e^(L_last - L_j) take_j k_j v_j^T is a matrix product, all chunks at once; (2) a walk over a row's chunks,
+// S <- e^(L_last) S + U, leaves the state in front of every chunk where U stood, and the row's last state in its slot; (3) a
+// chunk's read-outs are two products, (scores q_t . k_j times their weights) x values and (e^(L_t) q_t) x S_0, again all
+// chunks at once.  One more column behind the values, whose "value" is 1, carries the normaliser as in the scan.  All
+// operands are float32 in LDS and the products run on v_mfma_f32_16x16x4_f32; a workgroup of four wavefronts forms 64 x 64
+// results, a wavefront 32 x 32 of them.  An item is a (row, chunk): the grid has as many as the step could have at most,
+// and a workgroup finds its row by walking the rows' lengths.
+constexpr int MC = 64;                   // tokens a chunk
+constexpr int MC_A = 68;                 // row length in LDS of an operand read down its rows (a lane a row)
+constexpr int MC_B = 80;                 // ... of an operand read along its rows (a lane a column)
+
+__device__ __forceinline__ bool memory_item(int item, int rows, const int* __restrict__ row_len, int& row, int& chunk) {
+    int base = 0;
+    for (int r = 0; r < rows; ++r) {
+        const int count = row_len[r];
+        const int chunks = count > 0 ? (count + MC - 1) / MC : 0;
+        if (item < base + chunks) { row = r; chunk = item - base; return true; }
+        base += chunks;
+    }
+    return false;
+}
+
+// acc += A B over inner indices [0, inner) (a multiple of 4): A's (m, i) at a[m * MC_A + i], m counted from the wavefront's first row;
+// B's (i, n) at b[i * b_inner + n * b_column], n counted from the wavefront's first column.
+// acc[mi][ni][e] is the result at row 16 mi + 4 (lane / 16) + e, column 16 ni + lane % 16.
+typedef float mc_f4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void memory_product(mc_f4 (&acc)[2][2], const float* a, const float* b, int b_inner, int b_column, int inner, int lane) {
+    const int r = lane & 15, g = lane >> 4;
+    for (int i = 0; i < inner; i += 4) {
+        const float a0 = a[r * MC_A + i + g], a1 = a[(r + 16) * MC_A + i + g];
+        const float b0 = b[(i + g) * b_inner + r * b_column], b1 = b[(i + g) * b_inner + (r + 16) * b_column];
+        acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b1, acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b0, acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1, acc[1][1], 0, 0, 0);
+    }
+}
+
+// (1) sums[item][head][channel][column] = sum_j e^(L_last - L_j) take_j k_j[channel] value_j[column]; grid (items, heads,
+// blocks of 64 columns of value_dim + 1), 256 threads.  A = the weighted keys, read as [channel][token]; B = the values.
+template <typename T>
+__global__ __launch_bounds__(256) void memory_chunk_sums_kernel(const T* __restrict__ k, long k_stride, const T* __restrict__ v, long v_stride,
+                                                                const float* __restrict__ coef, const double* __restrict__ run,
+                                                                const int* __restrict__ row_start, const int* __restrict__ row_len, int rows,
+                                                                float* __restrict__ sums, int heads, int dim, int value_dim) {
+    __shared__ float s_k[MC * MC_A];                     // [channel][token]
+    __shared__ float s_v[MC * MC_B];                     // [token][column]
+    __shared__ float s_w[MC];
+    int row, chunk;
+    if (!memory_item(blockIdx.x, rows, row_len, row, chunk)) return;
+    const int head = blockIdx.y, column0 = blockIdx.z * 64, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = min(MC, row_len[row] - chunk * MC);
+    const size_t token0 = (size_t)row_start[row] + (size_t)chunk * MC;
+    const int ld = value_dim + 1;
+    if (tid < MC) {
+        float w = 0.f;
+        if (tid < n) {
+            const double last = run[(token0 + n - 1) * heads + head];
+            w = expf((float)(last - run[(token0 + tid) * heads + head])) * coef[((token0 + tid) * heads + head) * 2 + 1];
+        }
+        s_w[tid] = w;
+    }
+    for (int i = tid; i < MC * 64; i += 256) {
+        const int t = i >> 6, c = column0 + (i & 63);
+        float value = 0.f;
+        if (t < n) value = c < value_dim ? (float)v[(token0 + t) * v_stride + (size_t)head * value_dim + c] : (c == value_dim ? 1.f : 0.f);
+        s_v[t * MC_B + (i & 63)] = value;
+    }
+    const int mt = wave >> 1, nt = wave & 1;
+    const int inner = (n + 3) & ~3;
+    for (int slab = 0; slab < dim; slab += 64) {
+        __syncthreads();                                 // s_w is there; the slab before has been read
+        for (int i = tid; i < MC * 64; i += 256) {
+            const int t = i >> 6, c = i & 63;            // (neighbouring threads read neighbouring channels of one token)
+            float key = 0.f;
+            if (t < n && slab + c < dim) key = (float)k[(token0 + t) * k_stride + (size_t)head * dim + slab + c] * s_w[t];
+            s_k[c * MC_A + t] = key;
+        }
+        __syncthreads();
+        if (slab + mt * 32 >= dim || column0 + nt * 32 > value_dim) continue;
+        mc_f4 acc[2][2] = {};
+        memory_product(acc, s_k + mt * 32 * MC_A, s_v + nt * 32, MC_B, 1, inner, lane);
+        float* base = sums + (((size_t)blockIdx.x * heads + head) * dim) * ld;
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int channel = slab + mt * 32 + 16 * mi + 4 * (lane >> 4) + e, column = column0 + nt * 32 + 16 * ni + (lane & 15);
+                    if (channel < dim && column <= value_dim) base[(size_t)channel * ld + column] = acc[mi][ni][e];
+                }
+    }
+}
+
+// (2) grid (rows, heads, blocks of 256 numbers of a head's dim x (value_dim + 1)); a thread walks one number of the state
+// through the row's chunks.  The next chunk's sum is loaded before this chunk's place is overwritten.
+__global__ __launch_bounds__(256) void memory_chunk_carry_kernel(float* __restrict__ sums, const double* __restrict__ run, float* state, long state_stride,
+                                                                 const int* __restrict__ slots, const int* __restrict__ row_start,
+                                                                 const int* __restrict__ row_len, const int* __restrict__ row_ctx,
+                                                                 int heads, int dim, int value_dim) {
+    const int row = blockIdx.x, head = blockIdx.y;
+    const int count = row_len[row];
+    if (count <= 0) return;
+    const int ld = value_dim + 1;
+    const long e = (long)blockIdx.z * 256 + threadIdx.x;
+    if (e >= (long)dim * ld) return;
+    const int channel = (int)(e / ld), column = (int)(e - (long)channel * ld);
+    int base = 0;
+    for (int r = 0; r < row; ++r) base += row_len[r] > 0 ? (row_len[r] + MC - 1) / MC : 0;
+    const int chunks = (count + MC - 1) / MC, start = row_start[row];
+    float* slot = state + (size_t)slots[row] * state_stride;
+    float* mine = column < value_dim ? slot + ((size_t)head * dim + channel) * value_dim + column
+                                     : slot + (size_t)heads * dim * value_dim + (size_t)head * dim + channel;
+    float S = row_ctx[row] - count > 0 ? *mine : 0.f;
+    const size_t step = (size_t)heads * dim * ld;
+    float* place = sums + ((size_t)base * heads + head) * dim * ld + e;
+    float sum = *place;
+    for (int c = 0; c < chunks; ++c) {
+        const float next = c + 1 < chunks ? place[step] : 0.f;
+        const size_t last = (size_t)start + min(count, (c + 1) * MC) - 1;
+        const float keep = expf((float)run[last * heads + head]);
+        *place = S;
+        S = __builtin_fmaf(keep, S, sum);
+        sum = next;
+        place += step;
+    }
+    *mine = S;
+}
+
+// (3) out[t][head][column] = sum_(j <= t) (q_t . k_j) e^(L_t - L_j) take_j value_j[column] + e^(L_t) sum_channel q_t[channel] S_0[channel][column],
+// q scaled; the column behind the values goes to below[t][head][0].  grid and workgroup as in (1).
+template <typename T>
+__global__ __launch_bounds__(256) void memory_chunk_read_kernel(const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
+                                                                const T* __restrict__ v, long v_stride, const float* __restrict__ coef,
+                                                                const double* __restrict__ run, float q_scale,
+                                                                const int* __restrict__ row_start, const int* __restrict__ row_len,
+                                                                const int* __restrict__ row_ctx, int rows, const float* __restrict__ sums,
+                                                                float* __restrict__ out, float* __restrict__ below, int heads, int dim, int value_dim) {
+    __shared__ float s_q[MC * MC_A];                     // [token][channel]
+    __shared__ float s_k[MC * MC_A];                     // [token][channel]; then the weighted scores [token t][token j]
+    __shared__ float s_v[MC * MC_B];                     // [token or channel][column]
+    __shared__ double s_run[MC];
+    __shared__ float s_take[MC];
+    int row, chunk;
+    if (!memory_item(blockIdx.x, rows, row_len, row, chunk)) return;
+    const int head = blockIdx.y, column0 = blockIdx.z * 64, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int count = row_len[row];
+    const int n = min(MC, count - chunk * MC);
+    const size_t token0 = (size_t)row_start[row] + (size_t)chunk * MC;
+    const int ld = value_dim + 1;
+    const bool from_zero = chunk == 0 && row_ctx[row] - count == 0;      // nothing stands in front of the sequence's first chunk
+    if (tid < MC) {
+        s_run[tid] = tid < n ? run[(token0 + tid) * heads + head] : 0.0;
+        s_take[tid] = tid < n ? coef[((token0 + tid) * heads + head) * 2 + 1] : 0.f;
+    }
+    const int mt = wave >> 1, nt = wave & 1;
+    // the scores of the wavefront's 32 tokens t against 32 tokens j (nothing to do where every j lies behind every t)
+    mc_f4 scores[2][2] = {};
+    for (int slab = 0; slab < dim; slab += 64) {
+        __syncthreads();
+        for (int i = tid; i < MC * 64; i += 256) {
+            const int t = i >> 6, c = i & 63;
+            float query = 0.f, key = 0.f;
+            if (t < n && slab + c < dim) {
+                query = (float)q[(token0 + t) * q_stride + (size_t)head * dim + slab + c] * q_scale;
+                key = (float)k[(token0 + t) * k_stride + (size_t)head * dim + slab + c];
+            }
+            s_q[t * MC_A + c] = query;
+            s_k[t * MC_A + c] = key;
+        }
+        __syncthreads();
+        if (nt <= mt) memory_product(scores, s_q + mt * 32 * MC_A, s_k + nt * 32 * MC_A, 1, MC_A, min(64, (dim - slab + 3) & ~3), lane);
+    }
+    __syncthreads();                                     // everybody has read the keys: their place takes the weighted scores
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int t = mt * 32 + 16 * mi + 4 * (lane >> 4) + e, j = nt * 32 + 16 * ni + (lane & 15);
+                float weight = 0.f;
+                if (j <= t && t < n) weight = expf((float)(s_run[t] - s_run[j])) * s_take[j];
+                s_k[t * MC_A + j] = scores[mi][ni][e] * weight;
+            }
+    for (int i = tid; i < MC * 64; i += 256) {
+        const int t = i >> 6, c = column0 + (i & 63);
+        float value = 0.f;
+        if (t < n) value = c < value_dim ? (float)v[(token0 + t) * v_stride + (size_t)head * value_dim + c] : (c == value_dim ? 1.f : 0.f);
+        s_v[t * MC_B + (i & 63)] = value;
+    }
+    __syncthreads();
+    const bool wanted = column0 + nt * 32 <= value_dim;  // (uniform in a wavefront)
+    mc_f4 acc[2][2] = {};
+    if (wanted) memory_product(acc, s_k + mt * 32 * MC_A, s_v + nt * 32, MC_B, 1, (mt + 1) * 32, lane);
+    if (!from_zero) {
+        const float* before = sums + (((size_t)blockIdx.x * heads + head) * dim) * ld;
+        for (int slab = 0; slab < dim; slab += 64) {
+            __syncthreads();
+            for (int i = tid; i < MC * 64; i += 256) {
+                const int t = i >> 6, c = i & 63;        // queries [token][channel] times what the chunk's state has kept
+                float query = 0.f;
+                if (t < n && slab + c < dim)
+                    query = (float)q[(token0 + t) * q_stride + (size_t)head * dim + slab + c] * q_scale * expf((float)s_run[t]);
+                s_q[t * MC_A + c] = query;
+                const int channel = slab + t, column = column0 + c;      // the state's slab [channel][column]
+                s_v[t * MC_B + c] = (channel < dim && column <= value_dim) ? before[(size_t)channel * ld + column] : 0.f;
+            }
+            __syncthreads();
+            if (wanted) memory_product(acc, s_q + mt * 32 * MC_A, s_v + nt * 32, MC_B, 1, min(64, (dim - slab + 3) & ~3), lane);
+        }
+    }
+    if (!wanted) return;
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int t = mt * 32 + 16 * mi + 4 * (lane >> 4) + e, column = column0 + nt * 32 + 16 * ni + (lane & 15);
+                if (t >= n || column > value_dim) continue;
+                if (column < value_dim) out[(token0 + t) * heads * value_dim + (size_t)head * value_dim + column] = acc[mi][ni][e];
+                else below[((token0 + t) * heads + head) * 2] = acc[mi][ni][e];
+            }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void tanh_kernel(T* __restrict__ x, long n) {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -509,7 +771,7 @@ LSA_EXPORT int lsa_heads_norm_gate(int code, const float* x, const float* weight
 LSA_EXPORT int lsa_matrix_memory(int code, const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
                                  const float* gates, float cap, float q_scale, float* state, long state_stride, const int* slots,
                                  const int* row_start, const int* row_len, const int* row_ctx, float* coef, float* out, float* below,
-                                 int rows, int heads, int dim, int value_dim, hipStream_t stream) {
+                                 int rows, int heads, int dim, int value_dim, double* run, float* sums, int items, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (dim < 1 || dim > MOST_DIM || value_dim < 1 || heads < 1 || !(cap > 0.f) || state == nullptr || coef == nullptr || below == nullptr) return -1;
     if (state_stride < (long)heads * dim * value_dim + (long)heads * dim + heads) return -1;
@@ -518,7 +780,24 @@ LSA_EXPORT int lsa_matrix_memory(int code, const void* q, long q_stride, const v
     const size_t lds = sizeof(float) * ((size_t)2 * CHUNK * waves * dk + (size_t)CHUNK * 64 + CHUNK + (size_t)waves * CHUNK * 64);
     if (lds > (size_t)MOST_LDS) return -1;
     memory_gates_kernel<<<dim3(rows, heads), 64, 0, stream>>>(gates, cap, state, state_stride, (long)heads * dim * value_dim + (long)heads * dim,
-                                                              slots, row_start, row_len, row_ctx, coef, below, heads);
+                                                              slots, row_start, row_len, row_ctx, coef, below, heads, run);
+    if (run != nullptr) {
+        // in chunks: run [T][heads] and sums [items][heads][dim][value_dim + 1] are the caller's scratch memory; items is no
+        // less than the number of chunks of 64 tokens that the rows have together
+        if (sums == nullptr || items <= 0) return -1;
+        const dim3 chunk_grid(items, heads, (value_dim + 1 + 63) / 64);
+        const dim3 carry_grid(rows, heads, (unsigned)(((long)dim * (value_dim + 1) + 255) / 256));
+#define LSA_CHUNKED(T) do { \
+            memory_chunk_sums_kernel<T><<<chunk_grid, 256, 0, stream>>>((const T*)k, k_stride, (const T*)v, v_stride, coef, run, row_start, row_len, rows, \
+                                                                        sums, heads, dim, value_dim); \
+            memory_chunk_carry_kernel<<<carry_grid, 256, 0, stream>>>(sums, run, state, state_stride, slots, row_start, row_len, row_ctx, heads, dim, value_dim); \
+            memory_chunk_read_kernel<T><<<chunk_grid, 256, 0, stream>>>((const T*)q, q_stride, (const T*)k, k_stride, (const T*)v, v_stride, coef, run, q_scale, \
+                                                                        row_start, row_len, row_ctx, rows, sums, out, below, heads, dim, value_dim); \
+        } while (0)
+        if (code) LSA_CHUNKED(bf16_t); else LSA_CHUNKED(float);
+#undef LSA_CHUNKED
+        LSA_LAUNCH_CHECK();
+    }
     dim3 grid(rows, heads, (value_dim + 1 + 63) / 64);
 #define LSA_LAUNCH(T, DK) \
         matrix_memory_kernel<T, DK><<<grid, waves * 64, lds, stream>>>((const T*)q, q_stride, (const T*)k, k_stride, (const T*)v, v_stride, \

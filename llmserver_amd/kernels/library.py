@@ -31,7 +31,7 @@ _SIGNATURES = {
     "lsa_streams_update": [_P, c_int, c_int, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, _P],
     "lsa_activation": [c_int, _P, c_long, c_int, _P],
     "lsa_matrix_memory": [c_int, _P, c_long, _P, c_long, _P, c_long, _P, c_float, c_float, _P, c_long, _P, _P, _P, _P, _P, _P, _P,
-                          c_int, c_int, c_int, c_int, _P],
+                          c_int, c_int, c_int, c_int, _P, _P, c_int, _P],
     "lsa_norm_add_norm": [_P, _P, _P, c_int, c_float, c_float, _P, c_float, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_qkv_prepare": [c_int, _P, c_long, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                         _P, c_int, c_int, c_int, _P],

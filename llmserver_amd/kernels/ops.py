@@ -1198,10 +1198,33 @@ class HipOps(KernelNamespace):
 
     GATE_ACTIVATIONS = ("silu", "sigmoid")
 
+    MEMORY_CHUNK = 64           # tokens a chunk of the memory's chunked form (csrc/recurrent.hip)
+    MEMORY_CHUNKED_FROM = 64    # a step with this many tokens more than rows runs its memories in chunks
+
+    def matrix_memory_chunks(self, n_tokens, rows):
+        """How many chunks a step's rows can have at most if its memories are to run in chunks (matrix products over 64
+        tokens at a time, the states in front of the chunks walked between them), or 0 if they run token by token: steps
+        of one token a row, and steps that bring little more.  Decided from the step's shape alone, which the host knows
+        without asking the GPU."""
+        if n_tokens - rows < self.MEMORY_CHUNKED_FROM:
+            return 0
+        return n_tokens // self.MEMORY_CHUNK + rows
+
     def matrix_memory(self, q, k, v, gates, cap, q_scale, state, state_slots, row_start, row_len, row_ctx, out, below, coefficients,
-                      heads, dim, value_dim):
+                      heads, dim, value_dim, run=None, sums=None):
+        """``run`` (float64 [T, heads]) and ``sums`` (float32 [chunks, heads, dim, value_dim + 1]) are scratch memory of the
+        chunked form, both or neither; ``chunks`` is what :meth:`matrix_memory_chunks` said."""
         n = out.shape[0]
         rows = row_len.shape[0]
+        items = 0
+        if (run is None) != (sums is None):
+            raise ValueError("the chunked memory takes both of its scratch tensors")
+        if run is not None:
+            _check(run, "run", torch.float64, (n, heads))
+            items = sums.shape[0]
+            if items < n // self.MEMORY_CHUNK + rows:
+                raise ValueError(f"{items} chunks of scratch memory for {n} tokens in {rows} rows")
+            _check(sums, "sums", torch.float32, (items, heads, dim, value_dim + 1))
         lib = self._part_library("recurrent")
         if dim > lib.lsa_linear_recurrence_most_dim():
             raise ValueError(f"the memory kernel takes heads of up to {lib.lsa_linear_recurrence_most_dim()} key channels, got {dim}")
@@ -1218,7 +1241,7 @@ class HipOps(KernelNamespace):
         _launched(lib.lsa_matrix_memory(
             _code(q), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), _ptr(gates), float(cap), float(q_scale),
             pointer, stride, _ptr(state_slots), _ptr(row_start), _ptr(row_len), _ptr(row_ctx), _ptr(coefficients), _ptr(out), _ptr(below),
-            rows, heads, dim, value_dim, _stream()), "matrix_memory")
+            rows, heads, dim, value_dim, _ptr(run), _ptr(sums), items, _stream()), "matrix_memory")
 
     def heads_norm_gate(self, x, weight, weight_per_channel, eps, gate, out, heads, value_dim, gate_activation="silu", below=None, floor=0.0):
         n = x.shape[0]

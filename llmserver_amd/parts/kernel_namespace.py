@@ -100,8 +100,13 @@ class KernelNamespace:
         ``x / (max(|below[..., 0]|, below[..., 1]) + floor)``, a matrix memory's read-out under its normaliser."""
         raise NotImplementedError
 
+    def matrix_memory_chunks(self, n_tokens, rows):
+        """0: a step of this shape runs its matrix memories token by token.  Otherwise the memories run in chunks (matrix
+        products over a chunk's tokens) and want scratch memory for this many chunks (``matrix_memory``'s ``run``, ``sums``)."""
+        return 0
+
     def matrix_memory(self, q, k, v, gates, cap, q_scale, state, state_slots, row_start, row_len, row_ctx, out, below, coefficients,
-                      heads, dim, value_dim):
+                      heads, dim, value_dim, run=None, sums=None):
         """A matrix memory with exponential gates, per row (request) and head over the row's tokens in order, all float32.
         ``gates [T, 2 * heads]``: the input gates' logits, then the forget gates'.  ``i = cap * tanh(z_i / cap)``,
         ``f = logsigmoid(cap * tanh(z_f / cap))``, ``m_t = max(f + m_(t-1), i)``, ``keep = exp(f + m_(t-1) - m_t)``,
@@ -110,7 +115,9 @@ class KernelNamespace:
         (n_t . (q_t * q_scale), exp(-m_t))``, ``coefficients [T, heads, 2]`` scratch (keep, take).  ``q, k [T, heads * dim]``,
         ``v [T, heads * value_dim]`` (views with unit stride along a row).  ``state[slot]``: ``S [heads, dim, value_dim]``,
         then ``n [heads, dim]``, then ``m [heads]``; a row whose first token stands at position 0 starts from zeros whatever
-        the slot holds; the state after the row's last token is stored back."""
+        the slot holds; the state after the row's last token is stored back.  ``run`` (float64 ``[T, heads]``) and ``sums``
+        (float32 ``[chunks, heads, dim, value_dim + 1]``): scratch memory of the chunked form, given when
+        ``matrix_memory_chunks`` said so."""
         raise NotImplementedError
 
     # Several residual streams in 32-bit.

@@ -354,8 +354,14 @@ class MatrixMemory(Mixer):
         mixed = ctx.empty((n, values), dtype=torch.float32)
         below = ctx.empty((n, self.heads, 2), dtype=torch.float32)
         coefficients = ctx.empty((n, self.heads, 2), dtype=torch.float32)
+        # long portions run in chunks, as matrix products; the kernels then want scratch memory of the step's size
+        chunks = ops.matrix_memory_chunks(n, ctx.row_len.shape[0])
+        scratch = {}
+        if chunks:
+            scratch = {"run": ctx.empty((n, self.heads), dtype=torch.float64),
+                       "sums": ctx.empty((chunks, self.heads, self.dim, self.value_dim + 1), dtype=torch.float32)}
         ops.matrix_memory(q, k, v, gates, self.gate_cap, self.q_scale, cache.state, ctx.state_slots, ctx.row_start, ctx.row_len, ctx.row_ctx,
-                          mixed, below, coefficients, self.heads, self.dim, self.value_dim)
+                          mixed, below, coefficients, self.heads, self.dim, self.value_dim, **scratch)
         gated = ctx.empty((n, values))
         ops.heads_norm_gate(mixed, self.norm_weight, True, self.norm_eps, gate, gated, self.heads, self.value_dim, gate_activation="sigmoid",
                             below=below, floor=self.floor)

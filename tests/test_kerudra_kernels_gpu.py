@@ -63,17 +63,19 @@ def test_streams_start_read_and_update(ops, dtype, streams, width):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,dim,vdim,cap", [(3, 24, 40, 4.0), (2, 64, 64, 15.0), (5, 7, 100, 1.0), (1, 130, 9, 30.0), (2, 300, 65, 8.0),
                                                 (4, 128, 128, 15.0), (2, 48, 63, 15.0)])
-def test_matrix_memory_over_steps_and_slots(ops, dtype, heads, dim, vdim, cap):
+@pytest.mark.parametrize("chunked", [False, True])
+def test_matrix_memory_over_steps_and_slots(ops, dtype, heads, dim, vdim, cap, chunked):
     """Rows of unequal portions, an empty row, single tokens, portions longer than the kernel's chunks; a request that
-    starts again in a used slot starts from zeros (matrix, normaliser and maximum)."""
-    print(f"matrix_memory {dtype} {heads} {dim} {vdim} {cap}", flush=True)
+    starts again in a used slot starts from zeros (matrix, normaliser and maximum).  ``chunked``: every step in the
+    chunked form (chunks of one token up to whole ones, rows of several chunks)."""
+    print(f"matrix_memory {dtype} {heads} {dim} {vdim} {cap} chunked={chunked}", flush=True)
     twin = TorchOps()
     size = heads * dim * vdim + heads * dim + heads
     states = [torch.randn(4, size + 3, device="cuda") for _ in range(2)]
     states[1].copy_(states[0])
     slots = torch.tensor([2, 0, 3], dtype=torch.int32, device="cuda")
     firsts = [0, 0, 0]
-    for step, lengths in enumerate(([5, 1, 37], [1, 1, 1], [18, 0, 2], [1, 1, 1], [2, 140, 1])):
+    for step, lengths in enumerate(([5, 1, 37], [1, 1, 1], [18, 0, 2], [1, 1, 1], [2, 140, 1], [64, 65, 128], [200, 0, 3])):
         if step == 3:
             firsts[1] = 0                          # the second request ends; another one starts in its slot
         token_row, positions, row_start, row_len, row_ctx = batch(lengths, firsts, "cuda")
@@ -85,8 +87,14 @@ def test_matrix_memory_over_steps_and_slots(ops, dtype, heads, dim, vdim, cap):
         outs = [torch.zeros(n, heads * vdim, device="cuda") for _ in range(2)]
         belows = [torch.zeros(n, heads, 2, device="cuda") for _ in range(2)]
         coefs = [torch.zeros(n, heads, 2, device="cuda") for _ in range(2)]
+        scratch = {}
+        if chunked:
+            # (filled with what is no number: nothing may be read that has not been written)
+            scratch = {"run": torch.full((n, heads), float("nan"), device="cuda", dtype=torch.float64),
+                       "sums": torch.full((n // 64 + len(lengths), heads, dim, vdim + 1), float("nan"), device="cuda")}
         for which, state, out, below, coef in zip((ops, twin), states, outs, belows, coefs):
-            which.matrix_memory(q, k, v, gates, cap, dim ** -0.5, state, slots, row_start, row_len, row_ctx, out, below, coef, heads, dim, vdim)
+            which.matrix_memory(q, k, v, gates, cap, dim ** -0.5, state, slots, row_start, row_len, row_ctx, out, below, coef, heads, dim, vdim,
+                                **(scratch if which is ops else {}))
         close(coefs[0], coefs[1], torch.float32, f"coefficients, step {step}")
         close(outs[0], outs[1], torch.float32, f"read-out, step {step}")
         close(belows[0], belows[1], torch.float32, f"below, step {step}")
@@ -123,6 +131,39 @@ def test_a_memory_does_not_depend_on_how_its_tokens_are_cut(ops, dtype):
         results.append((out, below, state))
     for out, below, state in results[1:]:
         assert torch.equal(out, results[0][0]) and torch.equal(below, results[0][1]) and torch.equal(state, results[0][2])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_memory_in_chunks_equals_the_memory_token_by_token(ops, dtype):
+    """A prompt of 700 tokens beside two short rows, at the sizes of a real model's heads and from a state that is there:
+    the chunked form against the scan, read-outs, normalisers and states; then the step's shape decides by itself."""
+    heads, dim, vdim = 3, 128, 192
+    lengths, firsts = [700, 1, 90], [40, 7, 0]
+    n = sum(lengths)
+    _, _, row_start, row_len, row_ctx = batch(lengths, firsts, "cuda")
+    slots = torch.tensor([1, 2, 0], dtype=torch.int32, device="cuda")
+    proj = (0.5 * torch.randn(n, 2 * heads * dim + heads * vdim, device="cuda")).to(dtype)
+    q, k, v = proj[:, :heads * dim], proj[:, heads * dim:2 * heads * dim], proj[:, 2 * heads * dim:]
+    gates = 5 * torch.randn(n, 2 * heads, device="cuda")
+    gates[:, heads:] += 6.0
+    size = heads * dim * vdim + heads * dim + heads
+    start = torch.randn(3, size, device="cuda")
+    start[:, -heads:] = 0.5
+    results = []
+    for chunked in (False, True):
+        state = start.clone()
+        out, below, coef = torch.zeros(n, heads * vdim, device="cuda"), torch.zeros(n, heads, 2, device="cuda"), torch.zeros(n, heads, 2, device="cuda")
+        scratch = {}
+        if chunked:
+            chunks = ops.matrix_memory_chunks(n, len(lengths))
+            assert chunks >= sum(-(-length // 64) for length in lengths)
+            scratch = {"run": torch.empty(n, heads, device="cuda", dtype=torch.float64), "sums": torch.empty(chunks, heads, dim, vdim + 1, device="cuda")}
+        ops.matrix_memory(q, k, v, gates, 15.0, dim ** -0.5, state, slots, row_start, row_len, row_ctx, out, below, coef, heads, dim, vdim, **scratch)
+        results.append((out, below, state, coef))
+    assert torch.equal(results[0][3], results[1][3]) and torch.equal(results[0][1][..., 1], results[1][1][..., 1])     # the gates' walk is one
+    for index, what in enumerate(("read-out", "below", "state")):
+        close(results[1][index], results[0][index], torch.float32, what)
+    assert ops.matrix_memory_chunks(3, 3) == 0 and ops.matrix_memory_chunks(40, 3) == 0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

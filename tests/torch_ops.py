@@ -383,8 +383,11 @@ class TorchOps(KernelNamespace):
         g = torch.sigmoid(g) if gate_activation == "sigmoid" else g * torch.sigmoid(g)
         out.copy_((normed * g).reshape(n, heads * value_dim).to(out.dtype))
 
+    def matrix_memory_chunks(self, n_tokens, rows):
+        return 0
+
     def matrix_memory(self, q, k, v, gates, cap, q_scale, state, state_slots, row_start, row_len, row_ctx, out, below, coefficients,
-                      heads, dim, value_dim):
+                      heads, dim, value_dim, run=None, sums=None):
         matrix_size, normaliser_size = heads * dim * value_dim, heads * dim
         log_in = cap * torch.tanh(gates[:, :heads].float() / cap)
         log_forget = torch.nn.functional.logsigmoid(cap * torch.tanh(gates[:, heads:].float() / cap))
