@@ -225,67 +225,69 @@ __global__ __launch_bounds__(64) void heads_norm_gate_kernel(const float* __rest
 // ---- a matrix memory with exponential gates --------------------------------------------------------------------------
 // Per head and token: log input gate i = cap tanh(z_i / cap), log forget gate f = logsigmoid(cap tanh(z_f / cap)), a running
 // maximum m_t = max(f + m_(t-1), i) that starts at 0, and from them what the memory's update needs: keep = exp(f + m_(t-1) -
-// m_t), take = exp(i - m_t), and exp(-m_t) for the read-out's denominator.  grid (rows, heads), one wavefront: the row's
-// tokens in chunks of 64, a lane a token for the transcendental functions, one lane for the maximum's walk through the
-// chunk (two dependent instructions a token).  gates [T][2 heads] (inputs, then forgets), coef [T][heads][2] (keep, take),
+// m_t), take = exp(i - m_t), and exp(-m_t) for the read-out's denominator.  grid (rows, heads), eight wavefronts: the row's
+// tokens 512 at a time, a thread a token for the transcendental functions, one thread for the maximum's walk through them
+// (two dependent instructions a token).  gates [T][2 heads] (inputs, then forgets), coef [T][heads][2] (keep, take),
 // below [T][heads][2] (its second number is written here), top[slot][head] the maximum between steps (0 at position 0).
 // run (or nullptr) [T][heads]: the sum of log keep from the first token of a token's chunk of 64 (counted from the row's
 // first token of this step) up to the token itself, in 64-bit: what the chunked form of the memory forms its weights from.
-__global__ __launch_bounds__(64) void memory_gates_kernel(const float* __restrict__ gates, float cap, float* state, long state_stride,
+constexpr int GATES_WAVES = 8;
+__global__ __launch_bounds__(64 * GATES_WAVES) void memory_gates_kernel(const float* __restrict__ gates, float cap, float* state, long state_stride,
                                                           long top_offset, const int* __restrict__ slots, const int* __restrict__ row_start,
                                                           const int* __restrict__ row_len, const int* __restrict__ row_ctx,
                                                           float* __restrict__ coef, float* __restrict__ below, int heads,
                                                           double* __restrict__ run) {
-    __shared__ __align__(16) float s_in[64], s_forget[64], s_top[68];
-    const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    constexpr int GROUP = 64 * GATES_WAVES;                            // tokens at a time: a wavefront a chunk of 64
+    __shared__ __align__(16) float s_in[GROUP], s_forget[GROUP], s_top[GROUP + 4];
+    const int row = blockIdx.x, head = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
     const int count = row_len[row];
     if (count <= 0) return;
     const int start = row_start[row], first_position = row_ctx[row] - count;
     float* kept = state + (size_t)slots[row] * state_stride + top_offset + head;
-    float top = first_position > 0 ? *kept : 0.f;                      // (the same number in every lane)
+    float top = first_position > 0 ? *kept : 0.f;                      // (the same number in every thread)
     const float inv_cap = 1.f / cap;
-    for (int t0 = 0; t0 < count; t0 += 64) {
-        const int n = min(64, count - t0);
-        const size_t token = (size_t)(start + t0 + lane);
+    for (int t0 = 0; t0 < count; t0 += GROUP) {
+        const int n = min(GROUP, count - t0);
+        const size_t token = (size_t)(start + t0 + tid);
         float log_in = 0.f, log_forget = 0.f;
-        if (lane < n) {
+        if (tid < n) {
             log_in = cap * tanhf(gates[token * 2 * heads + head] * inv_cap);
             const float z = cap * tanhf(gates[token * 2 * heads + heads + head] * inv_cap);
             log_forget = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
         }
-        __syncthreads();                                               // the chunk before has been read
-        s_in[lane] = log_in;
-        s_forget[lane] = log_forget;
+        __syncthreads();                                               // the group before has been read
+        s_in[tid] = log_in;
+        s_forget[tid] = log_forget;
         __syncthreads();
-        if (lane == 0) {
+        if (tid == 0) {                                                // the walk: one thread, two dependent instructions a token
             float m = top;
             s_top[0] = m;
-            if (n == 64) {                                             // a whole chunk: all loads first, then the chain alone
+            int t = 0;
+            for (; t + 64 <= n; t += 64) {                             // a whole chunk: all loads first, then the chain alone
                 float fs[64], is[64], ms[64];
 #pragma unroll
                 for (int t4 = 0; t4 < 16; ++t4) {
-                    const float4 f4 = reinterpret_cast<const float4*>(s_forget)[t4], i4 = reinterpret_cast<const float4*>(s_in)[t4];
+                    const float4 f4 = reinterpret_cast<const float4*>(s_forget + t)[t4], i4 = reinterpret_cast<const float4*>(s_in + t)[t4];
                     fs[4 * t4] = f4.x; fs[4 * t4 + 1] = f4.y; fs[4 * t4 + 2] = f4.z; fs[4 * t4 + 3] = f4.w;
                     is[4 * t4] = i4.x; is[4 * t4 + 1] = i4.y; is[4 * t4 + 2] = i4.z; is[4 * t4 + 3] = i4.w;
                 }
 #pragma unroll
-                for (int t = 0; t < 64; ++t) {
-                    m = fmaxf(fs[t] + m, is[t]);
-                    ms[t] = m;
+                for (int u = 0; u < 64; ++u) {
+                    m = fmaxf(fs[u] + m, is[u]);
+                    ms[u] = m;
                 }
 #pragma unroll
-                for (int t = 0; t < 64; ++t) s_top[t + 1] = ms[t];
-            } else {
-                for (int t = 0; t < n; ++t) {
-                    m = fmaxf(s_forget[t] + m, s_in[t]);
-                    s_top[t + 1] = m;
-                }
+                for (int u = 0; u < 64; ++u) s_top[t + u + 1] = ms[u];
+            }
+            for (; t < n; ++t) {
+                m = fmaxf(s_forget[t] + m, s_in[t]);
+                s_top[t + 1] = m;
             }
         }
         __syncthreads();
         float log_keep = 0.f;
-        if (lane < n) {
-            const float before = s_top[lane], now = s_top[lane + 1];
+        if (tid < n) {
+            const float before = s_top[tid], now = s_top[tid + 1];
             log_keep = (log_forget + before) - now;
             coef[(token * heads + head) * 2] = expf(log_keep);
             coef[(token * heads + head) * 2 + 1] = expf(log_in - now);
@@ -298,11 +300,11 @@ __global__ __launch_bounds__(64) void memory_gates_kernel(const float* __restric
                 const double other = __shfl_up(total, step, 64);
                 if (lane >= step) total += other;
             }
-            if (lane < n) run[token * heads + head] = total;
+            if (tid < n) run[token * heads + head] = total;
         }
         top = s_top[n];
     }
-    if (lane == 0) *kept = top;
+    if (tid == 0) *kept = top;
 }
 
 // One token of one wavefront's DK channels of a matrix memory: S = keep S + k value (value: the token's value column times its
@@ -452,19 +454,50 @@ __device__ __forceinline__ bool memory_item(int item, int rows, const int* __res
     return false;
 }
 
-// acc += A B over inner indices [0, inner) (a multiple of 4): A's (m, i) at a[m * MC_A + i], m counted from the wavefront's first row;
-// B's (i, n) at b[i * b_inner + n * b_column], n counted from the wavefront's first column.
-// acc[mi][ni][e] is the result at row 16 mi + 4 (lane / 16) + e, column 16 ni + lane % 16.
+// acc += A B over inner indices [0, inner) (a multiple of 16; what lies behind an operand's end is zeros): A's (m, i) at
+// a[m * MC_A + i], m counted from the wavefront's first row; B's (i, n) at b[i * b_inner + n * b_column], n counted from the
+// wavefront's first column.  acc[mi][ni][e] is the result at row 16 mi + 4 (lane / 16) + e, column 16 ni + lane % 16.
+// Sixteen inner indices at a time: their sixteen LDS loads are issued before the first of their sixteen products.
 typedef float mc_f4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void memory_product(mc_f4 (&acc)[2][2], const float* a, const float* b, int b_inner, int b_column, int inner, int lane) {
     const int r = lane & 15, g = lane >> 4;
-    for (int i = 0; i < inner; i += 4) {
-        const float a0 = a[r * MC_A + i + g], a1 = a[(r + 16) * MC_A + i + g];
-        const float b0 = b[(i + g) * b_inner + r * b_column], b1 = b[(i + g) * b_inner + (r + 16) * b_column];
-        acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b1, acc[0][1], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b0, acc[1][0], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1, acc[1][1], 0, 0, 0);
+    const float* a0 = a + r * MC_A + g;
+    const float* a1 = a0 + 16 * MC_A;
+    const float* b0 = b + g * b_inner + r * b_column;
+    const float* b1 = b0 + 16 * b_column;
+    for (int i = 0; i < inner; i += 16) {
+        float x0[4], x1[4], y0[4], y1[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            x0[u] = a0[i + 4 * u]; x1[u] = a1[i + 4 * u];
+            y0[u] = b0[(i + 4 * u) * b_inner]; y1[u] = b1[(i + 4 * u) * b_inner];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(x0[u], y0[u], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(x0[u], y1[u], acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(x1[u], y0[u], acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(x1[u], y1[u], acc[1][1], 0, 0, 0);
+        }
+    }
+}
+
+// A chunk's values of 64 columns from column0 on, [token][column] in LDS: zeros behind the chunk's last token and behind the
+// column of ones that stands behind the values.  All of a thread's loads are issued before it stores.
+template <typename T>
+__device__ __forceinline__ void memory_stage_values(float* s_v, const T* __restrict__ v, long v_stride, size_t token0, int n, int head,
+                                                    int value_dim, int column0, int tid) {
+    T values[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        // (every load is of a place that is there, so that none stands under a condition and all are on their way together)
+        const int t = min(4 * j + (tid >> 6), n - 1), c = min(column0 + (tid & 63), value_dim - 1);
+        values[j] = v[(token0 + t) * v_stride + (size_t)head * value_dim + c];
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int t = 4 * j + (tid >> 6), c = column0 + (tid & 63);
+        s_v[t * MC_B + (tid & 63)] = t < n ? (c < value_dim ? (float)values[j] : (c == value_dim ? 1.f : 0.f)) : 0.f;
     }
 }
 
@@ -492,21 +525,21 @@ __global__ __launch_bounds__(256) void memory_chunk_sums_kernel(const T* __restr
         }
         s_w[tid] = w;
     }
-    for (int i = tid; i < MC * 64; i += 256) {
-        const int t = i >> 6, c = column0 + (i & 63);
-        float value = 0.f;
-        if (t < n) value = c < value_dim ? (float)v[(token0 + t) * v_stride + (size_t)head * value_dim + c] : (c == value_dim ? 1.f : 0.f);
-        s_v[t * MC_B + (i & 63)] = value;
-    }
+    memory_stage_values(s_v, v, v_stride, token0, n, head, value_dim, column0, tid);
     const int mt = wave >> 1, nt = wave & 1;
-    const int inner = (n + 3) & ~3;
+    const int inner = (n + 15) & ~15;
     for (int slab = 0; slab < dim; slab += 64) {
+        T keys[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int t = min(4 * j + (tid >> 6), n - 1), c = min(slab + (tid & 63), dim - 1);    // (neighbouring threads read neighbouring channels of one token)
+            keys[j] = k[(token0 + t) * k_stride + (size_t)head * dim + c];
+        }
         __syncthreads();                                 // s_w is there; the slab before has been read
-        for (int i = tid; i < MC * 64; i += 256) {
-            const int t = i >> 6, c = i & 63;            // (neighbouring threads read neighbouring channels of one token)
-            float key = 0.f;
-            if (t < n && slab + c < dim) key = (float)k[(token0 + t) * k_stride + (size_t)head * dim + slab + c] * s_w[t];
-            s_k[c * MC_A + t] = key;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int t = 4 * j + (tid >> 6), c = tid & 63;
+            s_k[c * MC_A + t] = (t < n && slab + c < dim) ? (float)keys[j] * s_w[t] : 0.f;
         }
         __syncthreads();
         if (slab + mt * 32 >= dim || column0 + nt * 32 > value_dim) continue;
@@ -573,7 +606,7 @@ __global__ __launch_bounds__(256) void memory_chunk_read_kernel(const T* __restr
     __shared__ float s_k[MC * MC_A];                     // [token][channel]; then the weighted scores [token t][token j]
     __shared__ float s_v[MC * MC_B];                     // [token or channel][column]
     __shared__ double s_run[MC];
-    __shared__ float s_take[MC];
+    __shared__ float s_take[MC], s_decay[MC];            // take_j; e^(L_t)
     int row, chunk;
     if (!memory_item(blockIdx.x, rows, row_len, row, chunk)) return;
     const int head = blockIdx.y, column0 = blockIdx.z * 64, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -585,24 +618,29 @@ __global__ __launch_bounds__(256) void memory_chunk_read_kernel(const T* __restr
     if (tid < MC) {
         s_run[tid] = tid < n ? run[(token0 + tid) * heads + head] : 0.0;
         s_take[tid] = tid < n ? coef[((token0 + tid) * heads + head) * 2 + 1] : 0.f;
+        s_decay[tid] = expf((float)s_run[tid]);
     }
     const int mt = wave >> 1, nt = wave & 1;
     // the scores of the wavefront's 32 tokens t against 32 tokens j (nothing to do where every j lies behind every t)
     mc_f4 scores[2][2] = {};
     for (int slab = 0; slab < dim; slab += 64) {
-        __syncthreads();
-        for (int i = tid; i < MC * 64; i += 256) {
-            const int t = i >> 6, c = i & 63;
-            float query = 0.f, key = 0.f;
-            if (t < n && slab + c < dim) {
-                query = (float)q[(token0 + t) * q_stride + (size_t)head * dim + slab + c] * q_scale;
-                key = (float)k[(token0 + t) * k_stride + (size_t)head * dim + slab + c];
-            }
-            s_q[t * MC_A + c] = query;
-            s_k[t * MC_A + c] = key;
+        T queries[16], keys[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int t = min(4 * j + (tid >> 6), n - 1), c = min(slab + (tid & 63), dim - 1);
+            queries[j] = q[(token0 + t) * q_stride + (size_t)head * dim + c];
+            keys[j] = k[(token0 + t) * k_stride + (size_t)head * dim + c];
         }
         __syncthreads();
-        if (nt <= mt) memory_product(scores, s_q + mt * 32 * MC_A, s_k + nt * 32 * MC_A, 1, MC_A, min(64, (dim - slab + 3) & ~3), lane);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int t = 4 * j + (tid >> 6), c = tid & 63;
+            const bool there = t < n && slab + c < dim;
+            s_q[t * MC_A + c] = there ? (float)queries[j] * q_scale : 0.f;
+            s_k[t * MC_A + c] = there ? (float)keys[j] : 0.f;
+        }
+        __syncthreads();
+        if (nt <= mt) memory_product(scores, s_q + mt * 32 * MC_A, s_k + nt * 32 * MC_A, 1, MC_A, min(64, (dim - slab + 15) & ~15), lane);
     }
     __syncthreads();                                     // everybody has read the keys: their place takes the weighted scores
 #pragma unroll
@@ -616,12 +654,7 @@ __global__ __launch_bounds__(256) void memory_chunk_read_kernel(const T* __restr
                 if (j <= t && t < n) weight = expf((float)(s_run[t] - s_run[j])) * s_take[j];
                 s_k[t * MC_A + j] = scores[mi][ni][e] * weight;
             }
-    for (int i = tid; i < MC * 64; i += 256) {
-        const int t = i >> 6, c = column0 + (i & 63);
-        float value = 0.f;
-        if (t < n) value = c < value_dim ? (float)v[(token0 + t) * v_stride + (size_t)head * value_dim + c] : (c == value_dim ? 1.f : 0.f);
-        s_v[t * MC_B + (i & 63)] = value;
-    }
+    memory_stage_values(s_v, v, v_stride, token0, n, head, value_dim, column0, tid);
     __syncthreads();
     const bool wanted = column0 + nt * 32 <= value_dim;  // (uniform in a wavefront)
     mc_f4 acc[2][2] = {};
@@ -629,18 +662,24 @@ __global__ __launch_bounds__(256) void memory_chunk_read_kernel(const T* __restr
     if (!from_zero) {
         const float* before = sums + (((size_t)blockIdx.x * heads + head) * dim) * ld;
         for (int slab = 0; slab < dim; slab += 64) {
-            __syncthreads();
-            for (int i = tid; i < MC * 64; i += 256) {
-                const int t = i >> 6, c = i & 63;        // queries [token][channel] times what the chunk's state has kept
-                float query = 0.f;
-                if (t < n && slab + c < dim)
-                    query = (float)q[(token0 + t) * q_stride + (size_t)head * dim + slab + c] * q_scale * expf((float)s_run[t]);
-                s_q[t * MC_A + c] = query;
-                const int channel = slab + t, column = column0 + c;      // the state's slab [channel][column]
-                s_v[t * MC_B + c] = (channel < dim && column <= value_dim) ? before[(size_t)channel * ld + column] : 0.f;
+            T queries[16];
+            float kept[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int t = 4 * j + (tid >> 6), c = tid & 63;          // queries [token][channel] times what the chunk's state has kept
+                queries[j] = q[(token0 + min(t, n - 1)) * q_stride + (size_t)head * dim + min(slab + c, dim - 1)];
+                const int channel = min(slab + t, dim - 1), column = min(column0 + c, value_dim);      // the state's slab [channel][column]
+                kept[j] = before[(size_t)channel * ld + column];
             }
             __syncthreads();
-            if (wanted) memory_product(acc, s_q + mt * 32 * MC_A, s_v + nt * 32, MC_B, 1, min(64, (dim - slab + 3) & ~3), lane);
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int t = 4 * j + (tid >> 6), c = tid & 63;
+                s_q[t * MC_A + c] = (t < n && slab + c < dim) ? (float)queries[j] * q_scale * s_decay[t] : 0.f;
+                s_v[t * MC_B + c] = (slab + t < dim && column0 + c <= value_dim) ? kept[j] : 0.f;
+            }
+            __syncthreads();
+            if (wanted) memory_product(acc, s_q + mt * 32 * MC_A, s_v + nt * 32, MC_B, 1, min(64, (dim - slab + 15) & ~15), lane);
         }
     }
     if (!wanted) return;
@@ -779,7 +818,7 @@ LSA_EXPORT int lsa_matrix_memory(int code, const void* q, long q_stride, const v
     recurrence_lds(dim, dk, waves);
     const size_t lds = sizeof(float) * ((size_t)2 * CHUNK * waves * dk + (size_t)CHUNK * 64 + CHUNK + (size_t)waves * CHUNK * 64);
     if (lds > (size_t)MOST_LDS) return -1;
-    memory_gates_kernel<<<dim3(rows, heads), 64, 0, stream>>>(gates, cap, state, state_stride, (long)heads * dim * value_dim + (long)heads * dim,
+    memory_gates_kernel<<<dim3(rows, heads), 64 * GATES_WAVES, 0, stream>>>(gates, cap, state, state_stride, (long)heads * dim * value_dim + (long)heads * dim,
                                                               slots, row_start, row_len, row_ctx, coef, below, heads, run);
     if (run != nullptr) {
         // in chunks: run [T][heads] and sums [items][heads][dim][value_dim + 1] are the caller's scratch memory; items is no
