@@ -219,12 +219,14 @@ __global__ __launch_bounds__(256) void streams_read_kernel(const float* __restri
         for (int s = 0; s < S; ++s) u += r[s] * row[(size_t)s * stream_stride + i];
         return u;
     };
-    float kept[STREAM_CACHE];
+    float kept[STREAM_CACHE], weights[STREAM_CACHE];
     float sq = 0.f;
 #pragma unroll
     for (int k = 0; k < STREAM_CACHE; ++k) {
         const int i = threadIdx.x + k * 256;
-        kept[k] = i < width ? summed(i) : 0.f;
+        const float u = summed(min(i, width - 1));       // (a load of a place that is there stands under no condition)
+        weights[k] = weight[min(i, width - 1)];          // (asked for now: behind the sum of squares nothing waits for memory)
+        kept[k] = i < width ? u : 0.f;
         sq += kept[k] * kept[k];
     }
     for (int i = threadIdx.x + STREAM_CACHE * 256; i < width; i += 256) {
@@ -236,7 +238,7 @@ __global__ __launch_bounds__(256) void streams_read_kernel(const float* __restri
 #pragma unroll
     for (int k = 0; k < STREAM_CACHE; ++k) {
         const int i = threadIdx.x + k * 256;
-        if (i < width) o[i] = (O)(kept[k] * inv * weight[i]);
+        if (i < width) o[i] = (O)(kept[k] * inv * weights[k]);
     }
     for (int i = threadIdx.x + STREAM_CACHE * 256; i < width; i += 256) o[i] = (O)(summed(i) * inv * weight[i]);
 }
@@ -279,13 +281,36 @@ __global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__
         }
         return u;
     };
-    float kept[STREAM_CACHE];
+    // the first STREAM_CACHE columns of a thread: every load is issued before the first store (a store to the streams would
+    // otherwise hold back the loads behind it, and a row of one token would wait for memory once a column), and every load
+    // is of a place that is there, so that none stands under a condition
+    float kept[STREAM_CACHE], olds[STREAM_CACHE][S], updates[STREAM_CACHE], weights[STREAM_CACHE];
     float sq = 0.f;
 #pragma unroll
     for (int k = 0; k < STREAM_CACHE; ++k) {
+        const int i = min((int)threadIdx.x + k * 256, width - 1);
+#pragma unroll
+        for (int s = 0; s < S; ++s) olds[k][s] = row[(size_t)s * stream_stride + i];
+        updates[k] = (float)yr[i];
+        weights[k] = next_read ? next_weight[i] : 0.f;    // (asked for now: behind the sum of squares nothing waits for memory)
+    }
+#pragma unroll
+    for (int k = 0; k < STREAM_CACHE; ++k) {
         const int i = threadIdx.x + k * 256;
-        kept[k] = i < width ? updated(i) : 0.f;
-        sq += kept[k] * kept[k];
+        float u = 0.f;
+        if (i < width) {
+#pragma unroll
+            for (int t = 0; t < S; ++t) {
+                float fresh = 0.f;
+#pragma unroll
+                for (int s = 0; s < S; ++s) fresh += m[s][t] * olds[k][s];
+                fresh += w[t] * updates[k];
+                row[(size_t)t * stream_stride + i] = fresh;
+                u += r[t] * fresh;
+            }
+        }
+        kept[k] = u;
+        sq += u * u;
     }
     for (int i = threadIdx.x + STREAM_CACHE * 256; i < width; i += 256) {
         const float u = updated(i);
@@ -297,7 +322,7 @@ __global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__
 #pragma unroll
     for (int k = 0; k < STREAM_CACHE; ++k) {
         const int i = threadIdx.x + k * 256;
-        if (i < width) o[i] = (R)(kept[k] * inv * next_weight[i]);
+        if (i < width) o[i] = (R)(kept[k] * inv * weights[k]);
     }
     for (int i = threadIdx.x + STREAM_CACHE * 256; i < width; i += 256) {
         float u = 0.f;
