@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256) void embedding_wide_kernel(const T* __restrict
 
 // ---- several residual streams x [S][T][W], float32 ------------------------------------------------------------------------
 constexpr int MOST_STREAMS = 8;
-constexpr int STREAM_CACHE = 8;           // elements of a row a thread keeps between the two passes (rows of up to 2,048 are read once)
+constexpr int STREAM_CACHE = 8;           // elements of a row a thread keeps between the two passes (rows of up to 2,048 are read once; sixteen gained nothing at 4,096 and cost a prompt a little)
 
 // The kernels below take the number of streams as a template parameter: the small per-stream arrays then live in registers
 // (indexed by a run-time count they would go to scratch memory, and a row of one token would wait for that).
@@ -224,6 +224,10 @@ __global__ __launch_bounds__(256) void streams_read_kernel(const float* __restri
 #pragma unroll
     for (int k = 0; k < STREAM_CACHE; ++k) {
         const int i = threadIdx.x + k * 256;
+        if (k * 256 >= width) {                          // (the same for the whole workgroup)
+            kept[k] = weights[k] = 0.f;
+            continue;
+        }
         const float u = summed(min(i, width - 1));       // (a load of a place that is there stands under no condition)
         weights[k] = weight[min(i, width - 1)];          // (asked for now: behind the sum of squares nothing waits for memory)
         kept[k] = i < width ? u : 0.f;
@@ -288,6 +292,12 @@ __global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__
     float sq = 0.f;
 #pragma unroll
     for (int k = 0; k < STREAM_CACHE; ++k) {
+        if (k * 256 >= width) {                          // (the same for the whole workgroup: narrow rows ask for nothing twice)
+#pragma unroll
+            for (int s = 0; s < S; ++s) olds[k][s] = 0.f;
+            updates[k] = weights[k] = 0.f;
+            continue;
+        }
         const int i = min((int)threadIdx.x + k * 256, width - 1);
 #pragma unroll
         for (int s = 0; s < S; ++s) olds[k][s] = row[(size_t)s * stream_stride + i];
