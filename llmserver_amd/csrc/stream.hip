@@ -224,10 +224,6 @@ __global__ __launch_bounds__(256) void streams_read_kernel(const float* __restri
 #pragma unroll
     for (int k = 0; k < STREAM_CACHE; ++k) {
         const int i = threadIdx.x + k * 256;
-        if (k * 256 >= width) {                          // (the same for the whole workgroup)
-            kept[k] = weights[k] = 0.f;
-            continue;
-        }
         const float u = summed(min(i, width - 1));       // (a load of a place that is there stands under no condition)
         weights[k] = weight[min(i, width - 1)];          // (asked for now: behind the sum of squares nothing waits for memory)
         kept[k] = i < width ? u : 0.f;
@@ -292,12 +288,6 @@ __global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__
     float sq = 0.f;
 #pragma unroll
     for (int k = 0; k < STREAM_CACHE; ++k) {
-        if (k * 256 >= width) {                          // (the same for the whole workgroup: narrow rows ask for nothing twice)
-#pragma unroll
-            for (int s = 0; s < S; ++s) olds[k][s] = 0.f;
-            updates[k] = weights[k] = 0.f;
-            continue;
-        }
         const int i = min((int)threadIdx.x + k * 256, width - 1);
 #pragma unroll
         for (int s = 0; s < S; ++s) olds[k][s] = row[(size_t)s * stream_stride + i];

@@ -338,52 +338,72 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
             group = np.repeat(cut_groups, tiles_of_group[cut_groups])            # a merge for every tile of every cut group
             j = np.arange(len(group)) - np.repeat(np.cumsum(tiles_of_group[cut_groups]) - tiles_of_group[cut_groups], tiles_of_group[cut_groups])
             merges = np.stack([of_row[group], starts[group] + j * tokens_per_tile, first[group] + j * ranges[group], ranges[group]], axis=1).tolist()
-    for row in range(len(row_len)):
-        n, ctx = int(row_len[row]), int(row_ctx[row])
-        first_pos = ctx - n
-        if per_workgroup and tiles_per_row[row] >= min_tiles:
-            continue
-        for tile in range(int(tiles_per_row[row])):
-            q0 = tile * tokens_per_tile
-            q1 = min(q0 + tokens_per_tile, n)
-            k_end = first_pos + q1                       # last query of the tile sees keys < k_end
-            k_begin = 0 if window is None else max(0, first_pos + q0 - window + 1)
-            n_keys = k_end - k_begin
-            splits = 1
-            if fixed_splits is not None:
-                splits = fixed_splits
-            elif waves_unsplit < target_waves:
-                splits = min(most_splits, max(1, target_waves // max(1, waves_unsplit)), max(1, n_keys // tuning.fewest_keys_per_split))
-            if splits <= 1:
-                items.append((row, q0, k_begin, k_end))
-                slots.append(-1)
-                continue
-            start = (k_begin // key_align) * key_align
-            per = -(-(k_end - start) // splits)
-            per = -(-per // key_align) * key_align        # at most `splits` items, each a multiple of key_align keys
-            first_slot = n_slots
-            count = 0
-            while start < k_end or (fixed_splits is not None and count < splits):
-                lo, hi = max(start, k_begin), min(start + per, k_end)
-                items.append((row, q0, lo, max(lo, hi)) if lo < k_end else (row, q0, k_end, k_end))
-                slots.append(-1 if merge_in_workgroup else n_slots)
-                n_slots += 0 if merge_in_workgroup else 1
-                count += 1
-                start += per
-            if not merge_in_workgroup:
-                merges.append((row, q0, first_slot, count))
+    # The other rows' tiles, all at once, in the order (row, tile, key range): a tile whose keys are not cut is one item
+    # without a slot; a tile with ``splits`` ranges of a multiple of key_align keys each gets that many items (with
+    # ``fixed_splits`` exactly, the last ones possibly empty; otherwise as many as hold keys) and, unless its workgroup
+    # merges them itself, consecutive slots and one merge.
+    rest = np.ones(len(row_len), dtype=bool)
+    if per_workgroup:
+        rest = tiles_per_row < min_tiles
+    rest_rows = np.flatnonzero(rest & (tiles_per_row > 0))
+    if len(rest_rows):
+        counts = tiles_per_row[rest_rows]
+        t_row = np.repeat(rest_rows, counts)
+        t_tile = np.arange(len(t_row)) - np.repeat(np.cumsum(counts) - counts, counts)
+        q0 = t_tile * tokens_per_tile
+        q1 = np.minimum(q0 + tokens_per_tile, row_len[t_row])
+        first_pos = (row_ctx - row_len)[t_row]
+        t_end = first_pos + q1                           # last query of the tile sees keys < t_end
+        t_begin = np.zeros_like(t_end) if window is None else np.maximum(0, first_pos + q0 - window + 1)
+        if fixed_splits is not None:
+            splits = np.full(len(t_row), int(fixed_splits), dtype=np.int64)
+        elif waves_unsplit < target_waves:
+            splits = np.minimum(min(most_splits, max(1, target_waves // max(1, waves_unsplit))),
+                                np.maximum(1, (t_end - t_begin) // tuning.fewest_keys_per_split))
+        else:
+            splits = np.ones(len(t_row), dtype=np.int64)
+        cut = splits > 1
+        start = (t_begin // key_align) * key_align
+        per = -(-(t_end - start) // np.maximum(splits, 1))
+        per = np.maximum(-(-per // key_align) * key_align, 1)      # at most `splits` items, each a multiple of key_align keys
+        if fixed_splits is not None:
+            count = np.where(cut, splits, 1)
+        else:
+            count = np.where(cut, np.maximum(-(-(t_end - start) // per), 0), 1)
+        entry = np.repeat(np.arange(len(t_row)), count)          # an entry for every item of every tile
+        e = np.arange(len(entry)) - np.repeat(np.cumsum(count) - count, count)
+        lo = np.maximum(start[entry] + e * per[entry], t_begin[entry])
+        hi = np.minimum(start[entry] + (e + 1) * per[entry], t_end[entry])
+        empty = lo >= t_end[entry]
+        lo = np.where(cut[entry], np.where(empty, t_end[entry], lo), t_begin[entry])
+        hi = np.where(cut[entry], np.where(empty, t_end[entry], np.maximum(lo, hi)), t_end[entry])
+        items = np.stack([t_row[entry], q0[entry], lo, hi], axis=1)
+        if merge_in_workgroup:
+            slots = np.full(len(entry), -1, dtype=np.int64)
+        else:
+            slotted = cut[entry]
+            numbers = n_slots + np.cumsum(slotted) - 1
+            slots = np.where(slotted, numbers, -1)
+            with_items = cut & (count > 0)
+            first_slot = n_slots + np.cumsum(np.where(cut, count, 0)) - np.where(cut, count, 0)
+            merges = np.concatenate([np.asarray(merges, dtype=np.int64).reshape(-1, 4),
+                                     np.stack([t_row[with_items], q0[with_items], first_slot[with_items], count[with_items]], axis=1)])
+            n_slots += int(np.where(cut, count, 0).sum())
+    items = np.asarray(items, dtype=np.int64).reshape(-1, 4)
+    slots = np.asarray(slots, dtype=np.int64).reshape(-1)
+    merges = np.asarray(merges, dtype=np.int64).reshape(-1, 4)
     if fixed_tiles is not None:
         if fixed_splits is None or len(tiles):
             raise ValueError("a plan is filled up to a number of tiles only where every tile gets a fixed number of key ranges")
         real = len(items) // fixed_splits
         if real < 1 or real > fixed_tiles:
             raise ValueError(f"the step's rows make {real} tiles, the shape it is filled up to holds {fixed_tiles}")
-        items += items[:fixed_splits] * (fixed_tiles - real)
-        slots += slots[:fixed_splits] * (fixed_tiles - real)
-        merges += merges[:1] * (fixed_tiles - real)
-        n_slots = fixed_tiles * fixed_splits if merges else 0
-    items = np.asarray(items, dtype=np.int32).reshape(-1, 4)
-    merges = np.asarray(merges, dtype=np.int32).reshape(-1, 4)
+        items = np.concatenate([items, np.tile(items[:fixed_splits], (fixed_tiles - real, 1))])
+        slots = np.concatenate([slots, np.tile(slots[:fixed_splits], fixed_tiles - real)])
+        merges = np.concatenate([merges, np.tile(merges[:1], (fixed_tiles - real, 1))])
+        n_slots = fixed_tiles * fixed_splits if len(merges) else 0
+    items = items.astype(np.int32)
+    merges = merges.astype(np.int32)
     tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 6)
     tiles = tiles[np.argsort(tiles[:, 2] - tiles[:, 3], kind="stable")]       # most keys first: the long tiles must not start last
     tile_slots = np.ascontiguousarray(tiles[:, 4:]) if len(tiles) and int(tiles[:, 4].max()) >= 0 else None
