@@ -226,71 +226,55 @@ __global__ __launch_bounds__(64) void heads_norm_gate_kernel(const float* __rest
 // Per head and token: log input gate i = cap tanh(z_i / cap), log forget gate f = logsigmoid(cap tanh(z_f / cap)), a running
 // maximum m_t = max(f + m_(t-1), i) that starts at 0, and from them what the memory's update needs: keep = exp(f + m_(t-1) -
 // m_t), take = exp(i - m_t), and exp(-m_t) for the read-out's denominator.  grid (rows, heads), eight wavefronts: the row's
-// tokens 512 at a time, a thread a token for the transcendental functions, one thread for the maximum's walk through them
-// (two dependent instructions a token).  gates [T][2 heads] (inputs, then forgets), coef [T][heads][2] (keep, take),
+// tokens 448 at a time; seven wavefronts have a thread a token for the transcendental functions, one thread of the eighth
+// walks the maximum through the tokens (two dependent instructions a token), and while it walks a group the others
+// prepare the group behind it and finish the group before it.  gates [T][2 heads] (inputs, then forgets), coef [T][heads][2] (keep, take),
 // below [T][heads][2] (its second number is written here), top[slot][head] the maximum between steps (0 at position 0).
 // run (or nullptr) [T][heads]: the sum of log keep from the first token of a token's chunk of 64 (counted from the row's
 // first token of this step) up to the token itself, in 64-bit: what the chunked form of the memory forms its weights from.
-constexpr int GATES_WAVES = 8;
+constexpr int GATES_WAVES = 8;            // the first walks, the others work: seven chunks of 64 tokens at a time
 __global__ __launch_bounds__(64 * GATES_WAVES) void memory_gates_kernel(const float* __restrict__ gates, float cap, float* state, long state_stride,
                                                           long top_offset, const int* __restrict__ slots, const int* __restrict__ row_start,
                                                           const int* __restrict__ row_len, const int* __restrict__ row_ctx,
                                                           float* __restrict__ coef, float* __restrict__ below, int heads,
                                                           double* __restrict__ run) {
-    constexpr int GROUP = 64 * GATES_WAVES;                            // tokens at a time: a wavefront a chunk of 64
-    __shared__ __align__(16) float s_in[GROUP], s_forget[GROUP], s_top[GROUP + 4];
+    constexpr int GROUP = 64 * (GATES_WAVES - 1);                      // tokens at a time: a working wavefront a chunk of 64
+    // two of each: while one group's maxima are walked, the group behind it is prepared and the group before it finished
+    __shared__ __align__(16) float s_in[2][GROUP], s_forget[2][GROUP], s_top[2][GROUP + 8];                 // (the maximum in front of a group's token t at [3 + t], behind it at [4 + t]: sixteen bytes at a time)
     const int row = blockIdx.x, head = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
     const int count = row_len[row];
     if (count <= 0) return;
     const int start = row_start[row], first_position = row_ctx[row] - count;
     float* kept = state + (size_t)slots[row] * state_stride + top_offset + head;
-    float top = first_position > 0 ? *kept : 0.f;                      // (the same number in every thread)
     const float inv_cap = 1.f / cap;
-    for (int t0 = 0; t0 < count; t0 += GROUP) {
-        const int n = min(GROUP, count - t0);
-        const size_t token = (size_t)(start + t0 + tid);
-        float log_in = 0.f, log_forget = 0.f;
-        if (tid < n) {
+    const int groups = (count + GROUP - 1) / GROUP;
+    const bool walker = tid < 64;
+    const int mine = tid - 64;                                         // a worker's token of a group
+    float m = 0.f;                                                     // (the walker's: the maximum so far)
+    if (tid == 0) m = first_position > 0 ? *kept : 0.f;
+    // what a worker keeps of its token of the group that is being walked, until the maxima are there
+    float log_in = 0.f, log_forget = 0.f;
+    auto prepare = [&](int g) {                                        // caps and logarithms of group g's gates
+        const int n = min(GROUP, count - g * GROUP);
+        log_in = 0.f; log_forget = 0.f;
+        if (mine < n) {
+            const size_t token = (size_t)(start + g * GROUP + mine);
             log_in = cap * tanhf(gates[token * 2 * heads + head] * inv_cap);
             const float z = cap * tanhf(gates[token * 2 * heads + heads + head] * inv_cap);
             log_forget = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
         }
-        __syncthreads();                                               // the group before has been read
-        s_in[tid] = log_in;
-        s_forget[tid] = log_forget;
-        __syncthreads();
-        if (tid == 0) {                                                // the walk: one thread, two dependent instructions a token
-            float m = top;
-            s_top[0] = m;
-            int t = 0;
-            for (; t + 64 <= n; t += 64) {                             // a whole chunk: all loads first, then the chain alone
-                float fs[64], is[64], ms[64];
-#pragma unroll
-                for (int t4 = 0; t4 < 16; ++t4) {
-                    const float4 f4 = reinterpret_cast<const float4*>(s_forget + t)[t4], i4 = reinterpret_cast<const float4*>(s_in + t)[t4];
-                    fs[4 * t4] = f4.x; fs[4 * t4 + 1] = f4.y; fs[4 * t4 + 2] = f4.z; fs[4 * t4 + 3] = f4.w;
-                    is[4 * t4] = i4.x; is[4 * t4 + 1] = i4.y; is[4 * t4 + 2] = i4.z; is[4 * t4 + 3] = i4.w;
-                }
-#pragma unroll
-                for (int u = 0; u < 64; ++u) {
-                    m = fmaxf(fs[u] + m, is[u]);
-                    ms[u] = m;
-                }
-#pragma unroll
-                for (int u = 0; u < 64; ++u) s_top[t + u + 1] = ms[u];
-            }
-            for (; t < n; ++t) {
-                m = fmaxf(s_forget[t] + m, s_in[t]);
-                s_top[t + 1] = m;
-            }
-        }
-        __syncthreads();
+        s_in[g & 1][mine] = log_in;
+        s_forget[g & 1][mine] = log_forget;
+    };
+    auto finish = [&](int g, float li, float lf) {                     // group g's coefficients, from its maxima
+        const int n = min(GROUP, count - g * GROUP);
+        const size_t token = (size_t)(start + g * GROUP + mine);
         float log_keep = 0.f;
-        if (tid < n) {
-            const float before = s_top[tid], now = s_top[tid + 1];
-            log_keep = (log_forget + before) - now;
+        if (mine < n) {
+            const float before = s_top[g & 1][3 + mine], now = s_top[g & 1][4 + mine];
+            log_keep = (lf + before) - now;
             coef[(token * heads + head) * 2] = expf(log_keep);
-            coef[(token * heads + head) * 2 + 1] = expf(log_in - now);
+            coef[(token * heads + head) * 2 + 1] = expf(li - now);
             below[(token * heads + head) * 2 + 1] = expf(-now);
         }
         if (run != nullptr) {                                          // the chunk's running sum of log keep, token by token
@@ -300,11 +284,53 @@ __global__ __launch_bounds__(64 * GATES_WAVES) void memory_gates_kernel(const fl
                 const double other = __shfl_up(total, step, 64);
                 if (lane >= step) total += other;
             }
-            if (tid < n) run[token * heads + head] = total;
+            if (mine < n) run[token * heads + head] = total;
         }
-        top = s_top[n];
+    };
+    if (!walker) prepare(0);
+    __syncthreads();
+    float walked_in = 0.f, walked_forget = 0.f;                        // a worker's token of the group that is being walked
+    for (int g = 0; g < groups; ++g) {
+        if (walker) {
+            if (tid == 0) {                                            // the walk: one thread, two dependent instructions a token
+                const int n = min(GROUP, count - g * GROUP);
+                const float* fs_all = s_forget[g & 1];
+                const float* is_all = s_in[g & 1];
+                float* tops = s_top[g & 1];
+                tops[3] = m;
+                int t = 0;
+                for (; t + 64 <= n; t += 64) {                         // a whole chunk: all loads first, then the chain alone
+                    float fs[64], is[64], ms[64];
+#pragma unroll
+                    for (int t4 = 0; t4 < 16; ++t4) {
+                        const float4 f4 = reinterpret_cast<const float4*>(fs_all + t)[t4], i4 = reinterpret_cast<const float4*>(is_all + t)[t4];
+                        fs[4 * t4] = f4.x; fs[4 * t4 + 1] = f4.y; fs[4 * t4 + 2] = f4.z; fs[4 * t4 + 3] = f4.w;
+                        is[4 * t4] = i4.x; is[4 * t4 + 1] = i4.y; is[4 * t4 + 2] = i4.z; is[4 * t4 + 3] = i4.w;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 64; ++u) {
+                        m = fmaxf(fs[u] + m, is[u]);
+                        ms[u] = m;
+                    }
+#pragma unroll
+                    for (int u4 = 0; u4 < 16; ++u4)
+                        reinterpret_cast<float4*>(tops + 4 + t)[u4] = make_float4(ms[4 * u4], ms[4 * u4 + 1], ms[4 * u4 + 2], ms[4 * u4 + 3]);
+                }
+                for (; t < n; ++t) {
+                    m = fmaxf(fs_all[t] + m, is_all[t]);
+                    tops[4 + t] = m;
+                }
+            }
+        } else {
+            const float li = walked_in, lf = walked_forget;            // (group g - 1's, whose maxima are there)
+            walked_in = log_in; walked_forget = log_forget;            // (group g's, which is being walked)
+            if (g + 1 < groups) prepare(g + 1);
+            if (g > 0) finish(g - 1, li, lf);
+        }
+        __syncthreads();
     }
-    if (tid == 0) *kept = top;
+    if (!walker) finish(groups - 1, walked_in, walked_forget);
+    if (tid == 0) *kept = m;
 }
 
 // One token of one wavefront's DK channels of a matrix memory: S = keep S + k value (value: the token's value column times its
