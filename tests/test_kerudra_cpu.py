@@ -19,7 +19,7 @@ from llmserver_amd.engine.replay import make_runner, replay
 from llmserver_amd.parts import PagedKVSpec, StateSpec
 from llmserver_amd.weights import build_model
 from tiny_kerudra import CASES, KA, KB, KC, KD, model_folder, plain_logits, plain_model
-from torch_ops import TorchOps
+from torch_ops import ChunkedMemoryOps, TorchOps
 
 
 def runner_for(case, max_tokens, page=None, live=4):
@@ -154,6 +154,22 @@ def test_prefill_equals_token_by_token_decoding_from_the_first_token(tmp_path):
     for case in ("KA", "KD"):
         requests = requests_of(case, (40,))
         check(case, run(case, traces.tail_decoded(requests, 64), tmp_path / case), requests)
+
+
+@pytest.mark.parametrize("case", ["KA", "KD"])
+@pytest.mark.parametrize("chunk", [5, 16, 64])
+def test_long_portions_through_the_chunked_form_of_the_memory(case, chunk, tmp_path):
+    """Steps that bring many tokens run their memories in chunks (products over a chunk's tokens, the state walked from
+    chunk to chunk), steps of single tokens as the scan; both leave the same state and logits, whatever the chunks' size
+    and wherever a portion ends: in the middle of a chunk, at its last token, one token into the next."""
+    requests = requests_of(case, (3 * chunk + 1, 2 * chunk, chunk - 1 if chunk > 2 else 2, 70))
+    steps = traces.changing_portions(requests, sizes=(chunk + 3, 2, 2 * chunk, 1, chunk))
+    ops = ChunkedMemoryOps(chunk=chunk, chunked_from=chunk // 2)
+    runner = make_runner(model_folder(case), "float32", traces.peak_tokens(steps), CASES[case][2], device="cpu", ops=ops, max_live=4)
+    replay(runner, traces.to_lines(steps).splitlines(), str(tmp_path), io.StringIO())
+    runner.cache.check_invariants()
+    assert ops.chunked_steps > 0
+    check(case, traces.collect(steps, str(tmp_path), CASES[case][0]["vocab"]), requests)
 
 
 @pytest.mark.parametrize("page", [4, 8, 64])

@@ -525,3 +525,74 @@ class TorchOps(KernelNamespace):
             target = float(uniform[row]) * float(running[-1])
             index = int(torch.searchsorted(running, torch.tensor(target, dtype=torch.float64), right=True))
             out[row] = min(index, logits.shape[1] - 1)
+
+
+class ChunkedMemoryOps(TorchOps):
+    """The twins, with the matrix memory in its chunked form where a step brings ``chunked_from`` tokens more than it has
+    rows: a row's tokens in chunks of ``chunk`` from its first token of the step; with ``L_t`` the sum of ``log keep`` from
+    the chunk's first token to ``t``, the read-outs are ``(Q K^T * W) V + e^(L_t) q_t S_0`` with
+    ``W[t, j] = e^(L_t - L_j) take_j`` for ``j <= t``, and the state behind the chunk is
+    ``e^(L_last) S_0 + sum_j e^(L_last - L_j) take_j k_j v_j^T``; a column of ones behind the values carries the normaliser."""
+
+    def __init__(self, chunk=64, chunked_from=64):
+        super().__init__()
+        self.chunk, self.chunked_from, self.chunked_steps = int(chunk), int(chunked_from), 0
+
+    def matrix_memory_chunks(self, n_tokens, rows):
+        return n_tokens // self.chunk + rows if n_tokens - rows >= self.chunked_from else 0
+
+    def matrix_memory(self, q, k, v, gates, cap, q_scale, state, state_slots, row_start, row_len, row_ctx, out, below, coefficients,
+                      heads, dim, value_dim, run=None, sums=None):
+        if run is None:
+            assert sums is None
+            return super().matrix_memory(q, k, v, gates, cap, q_scale, state, state_slots, row_start, row_len, row_ctx, out, below, coefficients,
+                                         heads, dim, value_dim)
+        n_tokens = out.shape[0]
+        assert tuple(run.shape) == (n_tokens, heads) and run.dtype == torch.float64
+        assert tuple(sums.shape[1:]) == (heads, dim, value_dim + 1) and sums.shape[0] >= n_tokens // self.chunk + len(row_len)
+        self.chunked_steps += 1
+        matrix_size, normaliser_size = heads * dim * value_dim, heads * dim
+        log_in = cap * torch.tanh(gates[:, :heads].float() / cap)
+        log_forget = torch.nn.functional.logsigmoid(cap * torch.tanh(gates[:, heads:].float() / cap))
+        item = 0
+        for row in range(len(row_len)):
+            start, count, end = int(row_start[row]), int(row_len[row]), int(row_ctx[row])
+            if count <= 0:
+                continue
+            slot = int(state_slots[row])
+            kept = state[slot].clone()
+            if end - count == 0:
+                kept.zero_()
+            both = torch.cat([kept[:matrix_size].view(heads, dim, value_dim),
+                              kept[matrix_size:matrix_size + normaliser_size].view(heads, dim, 1)], dim=-1)       # [h, d, v + 1]
+            top = kept[matrix_size + normaliser_size:matrix_size + normaliser_size + heads].clone()
+            for first in range(start, start + count, self.chunk):
+                tokens = slice(first, min(first + self.chunk, start + count))
+                size = tokens.stop - tokens.start
+                log_keep, take = torch.empty(size, heads), torch.empty(size, heads)
+                for t in range(size):                                       # the walk of the maximum, token by token
+                    new_top = torch.maximum(log_forget[first + t] + top, log_in[first + t])
+                    log_keep[t], take[t] = (log_forget[first + t] + top) - new_top, torch.exp(log_in[first + t] - new_top)
+                    below[first + t, :, 1] = torch.exp(-new_top)
+                    top = new_top
+                sums_of_logs = torch.cumsum(log_keep.double(), dim=0)                                  # L [C, h]
+                run[tokens] = sums_of_logs
+                coefficients[tokens, :, 0], coefficients[tokens, :, 1] = torch.exp(log_keep), take
+                queries = q[tokens].float().view(size, heads, dim) * q_scale
+                keys = k[tokens].float().view(size, heads, dim)
+                values = torch.cat([v[tokens].float().view(size, heads, value_dim), torch.ones(size, heads, 1)], dim=-1)
+                behind = torch.tril(torch.ones(size, size, dtype=torch.bool))[:, :, None]                # j <= t
+                apart = torch.where(behind, sums_of_logs[:, None, :] - sums_of_logs[None, :, :], torch.tensor(-float("inf"), dtype=torch.float64))
+                weights = torch.exp(apart.float()) * take[None, :, :]                                    # [t, j, h]
+                scores = torch.einsum("thd,jhd->tjh", queries, keys) * weights
+                sums[item] = both                                           # the state in front of the chunk
+                read = torch.einsum("tjh,jhv->thv", scores, values) \
+                    + torch.exp(sums_of_logs.float())[:, :, None] * torch.einsum("thd,hdv->thv", queries, both)
+                out[tokens] = read[..., :value_dim].reshape(size, -1)
+                below[tokens, :, 0] = read[..., value_dim]
+                to_last = torch.exp((sums_of_logs[-1][None, :] - sums_of_logs).float()) * take                           # [j, h]
+                both = torch.exp(sums_of_logs[-1].float())[:, None, None] * both + torch.einsum("jh,jhd,jhv->hdv", to_last, keys, values)
+                item += 1
+            state[slot, :matrix_size] = both[..., :value_dim].reshape(-1)
+            state[slot, matrix_size:matrix_size + normaliser_size] = both[..., value_dim].reshape(-1)
+            state[slot, matrix_size + normaliser_size:matrix_size + normaliser_size + heads] = top
