@@ -56,7 +56,7 @@ def _rotation_dict(dims: int, base: float) -> dict:
 
 @dataclasses.dataclass(frozen=True)
 class SharedValueAttentionSizes:
-    """Softmax attention with grouped key/value heads whose values are the keys as projected."""
+    """Softmax attention with grouped key/value heads without value weights: the unrotated key rows serve as values."""
     heads: int
     kv_heads: int
     dim: int

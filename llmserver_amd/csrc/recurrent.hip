@@ -224,7 +224,7 @@ __global__ __launch_bounds__(64) void heads_norm_gate_kernel(const float* __rest
 
 // ---- a matrix memory with exponential gates --------------------------------------------------------------------------
 // Per head and token: log input gate i = cap tanh(z_i / cap), log forget gate f = logsigmoid(cap tanh(z_f / cap)), a running
-// maximum m_t = max(f + m_(t-1), i) that starts at 0, and from them what the memory's update needs: keep = exp(f + m_(t-1) -
+// maximum m_t = max(f + m_(t-1), i) (0 in front of the first token), and from them what the memory's update needs: keep = exp(f + m_(t-1) -
 // m_t), take = exp(i - m_t), and exp(-m_t) for the read-out's denominator.  grid (rows, heads), eight wavefronts: the row's
 // tokens 448 at a time; seven wavefronts have a thread a token for the transcendental functions, one thread of the eighth
 // walks the maximum through the tokens (two dependent instructions a token), and while it walks a group the others

@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256) void streams_read_kernel(const float* __restri
     for (int i = threadIdx.x + STREAM_CACHE * 256; i < width; i += 256) o[i] = (O)(summed(i) * inv * weight[i]);
 }
 
-// All streams at once from the old ones, where they lie: x[t] <- sum_s mix[s][t] * x[s] + write[t] * y, and, where next_read
+// Every new stream from the streams as they stood before the update, stored where they lie: x[t] <- sum_s mix[s][t] * x[s] + write[t] * y, and, where next_read
 // is given, normed = rmsnorm(sum_t next_read[t] * x[t]) * next_weight: what the next sublayer reads, in the same pass (the
 // row of sums stays in registers between the two passes; wider rows are formed again from the streams just written, by the
 // thread that wrote them).  One workgroup a token row.

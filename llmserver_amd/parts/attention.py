@@ -477,7 +477,7 @@ class GQAttention(Mixer):
         ``softcap * tanh(score / softcap)`` (after the scale, before the mask), or None.  ``value_dim``: the size of a
         head's values if it is not the size of its queries and keys.  ``bare_names``: the names are the tensors' whole
         names (no ``.weight`` behind them; a bias is then named ``<matrix><bias_suffix>``).  ``values_are_keys``: there is
-        no value projection; a token's values are its keys as projected (bias included), before norm and rotation.
+        no value projection; a token's value row is what the key product left (bias included), taken before norm and rotation.
         ``names.qkv`` then names queries and keys only, and the stacked matrix gets the keys' rows a second time in
         the values' place when the tensors have been loaded, so every kernel sees queries, keys and values as usual.
 

@@ -265,7 +265,7 @@ class SandwichBlock(Block):
 
 class HyperConnection(Part):
     """How one sublayer is connected to ``streams`` residual streams ``x_1 .. x_S``.  It reads ``sum_s read[s] * x_s``; its
-    result ``y`` changes all streams at once, from the old ones: ``x_t <- sum_s mix[s, t] * x_s + mult * write[t] * y``
+    result ``y`` goes into every stream, each new stream formed from the streams as they stood before: ``x_t <- sum_s mix[s, t] * x_s + mult * write[t] * y``
     (``mix`` indexed [from, to]).  ``learned``: ``read``, ``write`` and ``mix`` are checkpoint tensors (``names``); not
     learned, they are ones and the identity, which is the plain residual sum ``x <- x + mult * y`` on one stream."""
 

@@ -127,7 +127,7 @@ class KernelNamespace:
         raise NotImplementedError
 
     def streams_update(self, streams, y, mix, write, next_read=None, next_weight=None, next_eps=0.0, normed=None):
-        """Where they lie, all streams at once from the old ones: ``streams[t] <- sum_s mix[s, t] * streams[s] + write[t] * y``
+        """Where they lie, every new stream from the streams as they stood before: ``streams[t] <- sum_s mix[s, t] * streams[s] + write[t] * y``
         (``y [T, W]`` of any type).  With ``next_read``: ``normed = rmsnorm(sum_t next_read[t] * streams[t]) * next_weight``
         of the new streams (eps ``next_eps``, any type)."""
         raise NotImplementedError

@@ -286,9 +286,9 @@ class MatrixMemoryNames:
 
 
 class MatrixMemory(Mixer):
-    """The matrix memory of xLSTM (mLSTM).  Per head, ``q = W_q h * dim^-1/2``, ``k``, ``v``; a log input gate
+    """A matrix-valued memory per head with exponential gates (the mLSTM cell).  Per head, ``q = W_q h * dim^-1/2``, ``k``, ``v``; a log input gate
     ``i = cap * tanh((W_i h + b_i) / cap)`` and a log forget gate ``f = logsigmoid(cap * tanh((W_f h + b_f) / cap))``.
-    With a running maximum ``m`` that starts at 0: ``m_t = max(f + m_(t-1), i)``, ``a = exp(f + m_(t-1) - m_t)``,
+    A stabiliser ``m`` (0 in front of the first token) keeps the exponentials in range: ``m_t = max(f + m_(t-1), i)``, ``a = exp(f + m_(t-1) - m_t)``,
     ``b = exp(i - m_t)``, ``S_t = a S_(t-1) + b k v^T``, ``n_t = a n_(t-1) + b k``,
     ``o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + floor)``.  Each head's ``o`` is divided by its root mean square, the
     heads side by side are multiplied by a weight per channel and by ``sigmoid(W_g h)``, then the output projection.

@@ -98,7 +98,7 @@ def rotation_of(sizes):
 
 
 def shared_value_attention(h, t, p, sizes, r=same):
-    """Grouped heads; the values are the keys as projected (bias included), before the rotation."""
+    """Grouped heads; value rows are the key product's rows (bias included), not rotated."""
     n, heads, dim = h.shape[0], sizes["heads"], sizes["dim"]
     groups = sizes.get("kv_heads", heads)
     q = r(h @ t[p + "q"].T + t[p + "q.b"]).view(n, heads, dim)
@@ -136,7 +136,7 @@ def capped(z, cap):
 
 
 def matrix_memory(h, t, p, sizes, eps, r=same, floor=1e-6):
-    """mLSTM: S and n per head under a running maximum m of the gates' logarithms that starts at 0."""
+    """mLSTM: S and n per head, kept in range by a stabiliser m (the largest log weight so far; 0 in front of the first token)."""
     n_tokens, heads, dim, vdim, cap = h.shape[0], sizes["heads"], sizes["dim"], sizes["vdim"], sizes["gate_cap"]
     q = r(h @ t[p + "q"].T).view(n_tokens, heads, dim) * dim ** -0.5
     k = r(h @ t[p + "k"].T).view(n_tokens, heads, dim)
@@ -182,7 +182,7 @@ def layer_runs(config):
 
 
 def connect(x, y, t, p, mult):
-    """Hyper-connection: every stream, all at once from the old ones, and the sublayer's result written into each."""
+    """Hyper-connection: each new stream is a mix of the streams as they stood before, plus its share of the sublayer's result."""
     return torch.einsum("st,snw->tnw", t[p + "mix"], x) + mult * t[p + "out"][:, None, None] * y[None]
 
 
