@@ -1,12 +1,13 @@
 from .base import ConfigError, ModelConfig, UnsupportedModelError, field, read_config_json
 from .named_sizes import NAMED_SIZES, named_config, named_size
 from .barotar import BarotarConfig
+from .gogalix import GogalixConfig
 from .kerudra import KerudraConfig
 from .qwen3 import Qwen3Config
 from .zepolix import ZepolixConfig
 from .registry import (config_from_dict, load_config, register_architecture, registered_architectures,
                        resolve_architecture, unregister_architecture)
 
-__all__ = ["ConfigError", "ModelConfig", "UnsupportedModelError", "field", "read_config_json", "Qwen3Config", "ZepolixConfig", "BarotarConfig", "KerudraConfig", "NAMED_SIZES", "named_config", "named_size",
+__all__ = ["ConfigError", "ModelConfig", "UnsupportedModelError", "field", "read_config_json", "Qwen3Config", "ZepolixConfig", "BarotarConfig", "KerudraConfig", "GogalixConfig", "NAMED_SIZES", "named_config", "named_size",
            "config_from_dict", "load_config", "register_architecture", "registered_architectures",
            "resolve_architecture", "unregister_architecture"]

@@ -1,8 +1,10 @@
 from .attention import AttentionNames, AttentionPlan, AttentionTuning, GQAttention, TileLaunchCost, build_attention_plan, group_tiling
 from .base import (INT_TABLE, MATRIX, VECTOR, Block, FeedForward, Mixer, Norm, PagedAndStateSpec, PagedKVSpec, ParamSpec, Part,
                    PositionEncoding, StateSpec)
-from .block import DepthAverage, HyperConnection, MultiStreamBlock, PostNormBlock, PreNormBlock, SandwichBlock
+from .block import DepthAverage, HyperConnection, MultiStreamBlock, ParallelGatedBlock, PostNormBlock, PreNormBlock, SandwichBlock
 from .conv import ShortConvolution
+from .delta import GatedDeltaNames, GatedDeltaRule
+from .differential import DifferentialAttention, DifferentialNames
 from .embedding import NormedTokenEmbedding, TokenEmbedding
 from .experts import RoutedExperts
 from .kernel_namespace import KernelNamespace
@@ -21,4 +23,5 @@ __all__ = ["KernelNamespace", "AttentionNames", "AttentionTuning", "TileLaunchCo
            "RotaryPosition", "PairedRotaryPosition", "PagedAndStateSpec", "DepthAverage", "PostNormBlock", "ShortConvolution",
            "NormedTokenEmbedding", "RoutedExperts", "LatentAttention", "LatentAttentionNames", "SandwichBlock", "ParallelMixers",
            "ScaledPair", "HyperConnection", "MultiStreamBlock", "PlainMLP", "StreamReadNorm", "MatrixMemory", "MatrixMemoryNames",
-           "GatedLinearAttention", "GatedLinearAttentionNames", "TimeMixing", "TimeMixingNames", "TokenShift"]
+           "GatedLinearAttention", "GatedLinearAttentionNames", "TimeMixing", "TimeMixingNames", "TokenShift", "ParallelGatedBlock",
+           "GatedDeltaRule", "GatedDeltaNames", "DifferentialAttention", "DifferentialNames"]

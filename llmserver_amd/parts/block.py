@@ -385,3 +385,88 @@ class MultiStreamBlock(Block):
             fed = self.ffn.forward(h, ctx)
             streams, normed = self._update(ctx, streams, fed, self.ffn_connection, following)
         return streams, (StreamUpdate(following, streams, normed=normed) if normed is not None else None)
+
+
+class ParallelGatedBlock(Block):
+    """Both sublayers read one norm of the stream and their results join it together:
+    ``h = norm(x)``, ``x <- x + s1 * sigmoid(G1 h + b1) * mixer(h) + s2 * sigmoid(G2 h + b2) * ffn(h)``, the stream in
+    32-bit throughout; ``ffn`` may be None.  ``s`` are per-channel scales, ``G``, ``b`` a gate per channel and sublayer
+    (both gates are one product).  The gates' sigmoids, the scales, the sum with the stream and the norm in front of the
+    next block are one kernel (``ops.gated_pair_update``).
+
+    ``names``: the checkpoint's names of the norm, the mixer, the feed-forward, the two scales and the two gates (a
+    gate's bias is its name with ``bias_suffix`` behind it)."""
+    takes_following = True
+
+    def __init__(self, norm: Norm, mixer: Mixer, ffn=None, names=("norm1", "mix", "mlp", "ls1", "ls2", "rg1", "rg2"), bias_suffix: str = ".b"):
+        from .linear import Linear
+        self.norm, self.mixer, self.ffn = norm, mixer, ffn
+        self.names = tuple(names)
+        self.width = norm.width
+        gate_names = self.names[5:7] if ffn is not None else self.names[5:6]
+        self.gates = Linear(self.width, gate_names, (self.width,) * len(gate_names), bias=True, bare_names=True, bias_suffix=bias_suffix)
+        self.scale1 = self.scale2 = None
+
+    def _parts(self):
+        norm, mix, mlp = self.names[:3]
+        parts = {norm: self.norm, mix: self.mixer}
+        if self.ffn is not None:
+            parts[mlp] = self.ffn
+        return parts
+
+    def _scale_names(self):
+        return self.names[3:5] if self.ffn is not None else self.names[3:4]
+
+    def param_specs(self):
+        specs = {f"{prefix}.{name}" if name else prefix: spec for prefix, part in self._parts().items()
+                 for name, spec in part.param_specs().items()}
+        specs.update(self.gates.param_specs())
+        for name in self._scale_names():
+            specs[name] = ParamSpec((self.width,), VECTOR, "norm")
+        return specs
+
+    def assign(self, name, tensor):
+        if name in self._scale_names():
+            if name == self.names[3]:
+                self.scale1 = tensor
+            else:
+                self.scale2 = tensor
+            return
+        if self.gates.owns(name):
+            self.gates.assign(name, tensor)
+            return
+        parts = self._parts()
+        if name in parts:                                   # the part's name is the tensor's
+            parts[name].assign("", tensor)
+            return
+        prefix, rest = name.split(".", 1)
+        parts[prefix].assign(rest, tensor)
+
+    def finalize(self):
+        self.gates.finalize()
+        for part in self._parts().values():
+            part.finalize()
+
+    def entry_norm(self):
+        return self.norm
+
+    def forward(self, resid, delta, ctx, cache, following=None):
+        """``delta``: None, or a :class:`StreamUpdate` whose ``normed`` rows are the stream under this block's norm (the
+        block before was told that norm as its ``following`` and has carried it out).  The stream is updated where it lies."""
+        x, h = resid, None
+        if isinstance(delta, StreamUpdate):
+            x = delta.resid
+            h = delta.normed if delta.norm is self.norm else None
+        elif delta is not None:
+            raise ValueError("this block takes a stream to which everything has been added")
+        if h is None:
+            h = ctx.empty(x.shape)
+            ctx.ops.norm_rows(x, None, self.norm.weight, self.norm.eps, h)
+        gates = self.gates.forward(h, ctx)
+        mixed = self.mixer.forward(h, ctx, cache)
+        fed = self.ffn.forward(h, ctx) if self.ffn is not None else None
+        following = SandwichBlock._same_kind(following)
+        normed = ctx.empty(x.shape) if following is not None else None
+        ctx.ops.gated_pair_update(x, gates, mixed, self.scale1, fed, self.scale2, following.weight if following is not None else None,
+                                  following.eps if following is not None else 0.0, normed)
+        return x, (StreamUpdate(following, x, normed=normed) if normed is not None else None)

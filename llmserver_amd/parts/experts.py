@@ -1,6 +1,6 @@
 """Routed experts: every token's feed-forward is a weighted sum of ``top`` of ``experts`` small gated feed-forwards.
 
-Router logits ``z = R h`` in 32-bit.  ``scoring="softmax"``: the ``top`` largest logits are chosen (the first of equal
+Router logits ``z = R h`` (plus a bias per expert, where the checkpoint has one) in 32-bit.  ``scoring="softmax"``: the ``top`` largest logits are chosen (the first of equal
 ones) and weighted by the softmax over the chosen logits only.  ``scoring="sigmoid"``: scores ``sigmoid(z)``; with
 ``groups=(count, keep)`` the experts form ``count`` equal groups of neighbours, a group's score is the sum of its two
 largest scores, and only experts of the ``keep`` best groups can be chosen; the ``top`` largest scores are chosen and
@@ -24,7 +24,7 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, width: int, intermediate: int, experts: int, top: int, router: str = "router", expert: str = "e{}",
                  pieces=("gate", "up", "down"), scoring: str = "softmax", groups=None, activation: str = "silu", limit: float = 0.0,
-                 reads_stream: bool = True):
+                 reads_stream: bool = True, router_bias: str = None):
         if not 1 <= top <= experts:
             raise ValueError(f"a token uses {top} of {experts} experts")
         if scoring not in self.SCORINGS or activation not in self.ACTIVATIONS:
@@ -40,6 +40,8 @@ class RoutedExperts(FeedForward):
         self.width, self.intermediate, self.experts, self.top = width, intermediate, experts, top
         self.router_name, self.expert_name, self.pieces = router, expert, tuple(pieces)
         self._parts = {}
+        self.router_bias_name = router_bias       # the name of a vector that is added to the router's logits, or None
+        self.router_bias = None   # float32 [experts]
         self.router = None        # float32 [experts, W]
         self.gate_up = None       # [experts, 2F, W]
         self.down = None          # [experts, W, F]
@@ -53,6 +55,8 @@ class RoutedExperts(FeedForward):
     def param_specs(self):
         share = self.top / self.experts
         specs = {self.router_name: ParamSpec((self.experts, self.width), VECTOR, "normal")}
+        if self.router_bias_name is not None:
+            specs[self.router_bias_name] = ParamSpec((self.experts,), VECTOR, "bias")
         for _, gate, up, down in self._names():
             specs[gate] = ParamSpec((self.intermediate, self.width), share_per_token=share)
             specs[up] = ParamSpec((self.intermediate, self.width), share_per_token=share)
@@ -62,6 +66,8 @@ class RoutedExperts(FeedForward):
     def assign(self, name, tensor):
         if name == self.router_name:
             self.router = tensor
+        elif name == self.router_bias_name:
+            self.router_bias = tensor
         else:
             self._parts[name] = tensor
 
@@ -79,6 +85,8 @@ class RoutedExperts(FeedForward):
         chosen = ctx.empty((n, self.top), dtype=torch.int32)
         weights = ctx.empty((n, self.top), dtype=torch.float32)
         extra = {} if self.scoring == "softmax" else {"scoring": self.scoring, "groups": self.groups}
+        if self.router_bias is not None:
+            extra["bias"] = self.router_bias
         ops.route_experts(x if stream is None else stream, self.router, self.top, chosen, weights, **extra)
         out = ctx.empty((n, self.width), dtype=torch.float32)
         extra = {} if self.activation == "silu" else {"activation": self.activation, "limit": self.limit}

@@ -196,12 +196,52 @@ class KernelNamespace:
         ``mixed [T, heads * row]``, ``up_values [heads, rank, v]`` given: ``y[h, t] = mixed[t, h, :rank] @ up_values[h]`` is made here."""
         raise NotImplementedError
 
+    # A block whose sublayers' results join the stream together under sigmoid gates.
+    def gated_pair_update(self, x, gates, y1, scale1, y2, scale2, next_weight=None, next_eps=0.0, normed=None):
+        """``x += scale1 * sigmoid(gates[:, :W]) * y1 + scale2 * sigmoid(gates[:, W:]) * y2`` in float32, where it lies
+        (``y2``, ``scale2`` None: one sublayer, ``gates [T, W]``); ``y`` of any type; with ``next_weight``:
+        ``normed = rmsnorm(x) * next_weight`` (eps ``next_eps``, any type)."""
+        raise NotImplementedError
+
+    # Differential attention: the two maps' results behind the attention kernels.
+    def differential_heads(self, attended, lam, keep, eps, out, kv_heads, group, value_dim, row):
+        """``attended [T, kv_heads * 2 * group * row]``: for key/value head ``g`` the results of map 1 of its ``group`` query
+        heads, then of map 2, each in a row of ``row`` numbers of which ``value_dim`` count.  ``out[t, (g * group + r) *
+        value_dim + j] = d / sqrt(mean_j(d^2) + eps) * keep`` with ``d = a1 - lam * a2``."""
+        raise NotImplementedError
+
+    # The gated delta rule.
+    def delta_prepare(self, proj, taps, state, offset, state_slots, token_row, positions, row_start, out, kv_heads, heads, dim,
+                      value_dim, q_scale, unit_eps, keep=False):
+        """The first ``C = 2 * kv_heads * dim + heads * value_dim`` columns of ``proj`` (queries, keys, values) pass a causal
+        convolution over each request's tokens per channel (``taps [C, K]``, tap ``j`` on the token ``K - 1 - j`` places
+        back, zeros before the sequence, earlier steps' inputs from ``state[slot, offset:]`` as ``[K - 1, C]``, oldest first)
+        and silu; every query and key head is then divided by ``sqrt(sum of its squares + unit_eps)``, queries also times
+        ``q_scale``.  ``out [T, C]`` float32.  ``keep`` (steps of one token per row only): the state also moves on by the
+        step's token, as :meth:`delta_conv_keep` would do."""
+        raise NotImplementedError
+
+    def delta_conv_keep(self, proj, channels, taps, state, offset, state_slots, row_start, row_len, row_ctx):
+        """Move every row's last ``taps - 1`` inputs of the convolutions (the step's, and the state's where the step brings
+        fewer) into ``state[slot, offset:]``."""
+        raise NotImplementedError
+
+    def delta_rule(self, prepared, strength, decay, decay_scale, decay_bias, per_channel, state, offset, state_slots, row_start,
+                   row_len, row_ctx, out, heads, kv_heads, dim, value_dim):
+        """Per head ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` over each row's tokens, with
+        ``prepared [T, C]`` from :meth:`delta_prepare` (head ``h`` reads query/key head ``h // (heads / kv_heads)``),
+        ``beta = sigmoid(strength[t, h])``, ``g = exp(-exp(decay_scale[h]) * softplus(decay + decay_bias))`` with ``decay [T,
+        heads]`` and ``decay_bias [heads]``, or, ``per_channel``, ``decay [T, heads * dim]`` float32 and ``decay_bias [heads *
+        dim]``: a decay for every row of ``S``.  ``S [heads, dim, value_dim]`` float32 lives in ``state[slot, offset:]``, zeros
+        before a sequence's first token.  ``out [T, heads * value_dim]`` float32."""
+        raise NotImplementedError
+
     # Routed experts.
-    def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None):
+    def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None, bias=None):
         """Float32 logits ``x router^T``; ``chosen [T, top]`` the largest (first of equals), ``weights`` their softmax.
         ``scoring="sigmoid"``: scores ``sigmoid(logits)``, the largest scores chosen, the scores themselves the weights;
         ``groups=(count, keep)``: only experts of the ``keep`` best of ``count`` equal groups of neighbours can be chosen,
-        a group's score the sum of its two largest scores (the first of equal groups)."""
+        a group's score the sum of its two largest scores (the first of equal groups).  ``bias [experts]`` joins the logits."""
         raise NotImplementedError
 
     def experts_gate_up(self, x, gate_up, chosen, hidden, activation="silu", limit=0.0):

@@ -31,8 +31,9 @@ class GatedMLP(FeedForward):
     ACTIVATIONS = {"silu": "silu", "swish": "silu", "gelu_tanh": "gelu_tanh", "gelu_pytorch_tanh": "gelu_tanh"}
 
     def __init__(self, width: int, intermediate: int, activation: str = "silu", bias: bool = False,
-                 names: GatedMLPNames = GatedMLPNames(), bare_names: bool = False):
-        """``bare_names``: the names are the tensors' whole names below the layer's (no ``.weight`` behind them)."""
+                 names: GatedMLPNames = GatedMLPNames(), bare_names: bool = False, bias_suffix: str = ""):
+        """``bare_names``: the names are the tensors' whole names below the layer's (no ``.weight`` behind them; a bias
+        is then named ``<matrix><bias_suffix>``)."""
         if activation not in self.ACTIVATIONS:
             raise ValueError(f"Unsupported activation {activation!r}; supported: {sorted(self.ACTIVATIONS)}")
         self.activation = self.ACTIVATIONS[activation]
@@ -43,17 +44,17 @@ class GatedMLP(FeedForward):
         self.names = names
         self.bare_names = bare_names
         self.gate_up = Linear(width, names.gate_up, (intermediate, intermediate) if len(names.gate_up) == 2 else (2 * intermediate,), bias,
-                              bare_names=bare_names)
-        self.down = Linear(intermediate, (names.down,), (width,), bias, bare_names=bare_names)
+                              bare_names=bare_names, bias_suffix=bias_suffix)
+        self.down = Linear(intermediate, (names.down,), (width,), bias, bare_names=bare_names, bias_suffix=bias_suffix)
 
     def param_specs(self):
         return {**self.gate_up.param_specs(), **self.down.param_specs()}
 
     def assign(self, name, tensor):
         owner = name if self.bare_names else name.rsplit(".", 1)[0]
-        if owner == self.names.down:
+        if owner == self.names.down or self.down.owns(name):
             self.down.assign(name, tensor)
-        elif owner in self.names.gate_up:
+        elif owner in self.names.gate_up or self.gate_up.owns(name):
             self.gate_up.assign(name, tensor)
         else:
             raise KeyError(name)

@@ -15,10 +15,13 @@ class RMSNorm(Norm):
     is stored around zero).  The sum is formed once, in 32-bit, when the tensor has been loaded, so every kernel sees a
     plain weight.  ``tensor``: the weight's name below the part's own ("" if the part's name is the tensor's).  ``scale``:
     a constant that multiplies the result (a model whose logits are a multiple of the head's product of the normed rows
-    says so here); it joins the weight in 32-bit when the tensor has been loaded."""
+    says so here); it joins the weight in 32-bit when the tensor has been loaded.  ``single``: the checkpoint holds one
+    number that multiplies every coordinate; it is spread over the width when it has been loaded, so every kernel sees a
+    plain weight."""
 
-    def __init__(self, width: int, eps: float, offset: float = 0.0, tensor: str = "weight", scale: float = 1.0):
+    def __init__(self, width: int, eps: float, offset: float = 0.0, tensor: str = "weight", scale: float = 1.0, single: bool = False):
         self.width = width
+        self.single = bool(single)
         self.eps = float(eps)
         self.offset = float(offset)
         self.scale = float(scale)
@@ -26,10 +29,12 @@ class RMSNorm(Norm):
         self.weight = None  # float32 [width], the offset added and the scale multiplied in
 
     def param_specs(self):
-        return {self.tensor: ParamSpec((self.width,), VECTOR, "bias" if self.offset else "norm")}
+        return {self.tensor: ParamSpec(() if self.single else (self.width,), VECTOR, "bias" if self.offset else "norm")}
 
     def assign(self, name, tensor):
         assert name == self.tensor
+        if self.single:
+            tensor = tensor.reshape(1).expand(self.width).contiguous()
         self.weight = tensor + self.offset if self.offset else tensor
         if self.scale != 1.0:
             self.weight = self.weight * self.scale

@@ -281,11 +281,15 @@ class TorchOps(KernelNamespace):
 
     # -- general preparation of queries, keys and values -------------------------------------------------
     def qkv_prepare(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
-                    n_q, n_kv, dim, value_dim, out_q, write_cache=True, pairing="neighbours"):
+                    n_q, n_kv, dim, value_dim, out_q, write_cache=True, pairing="neighbours", value_share=1):
         n, width = qkv.shape[0], keys.shape[-1]
         q = qkv[:, :n_q * dim].float().view(n, n_q, dim)
+        if not write_cache and qkv.shape[1] == n_q * dim:            # a layer that reads another's pages brings queries only
+            out_q.copy_(torch.nn.functional.pad(q, (0, width - dim)).reshape(n, n_q * width).to(out_q.dtype))
+            assert q_weight is None and cos_sin is None
+            return
         k = qkv[:, n_q * dim:(n_q + n_kv) * dim].float().view(n, n_kv, dim)
-        v = qkv[:, (n_q + n_kv) * dim:].float().view(n, n_kv, value_dim)
+        v = qkv[:, (n_q + n_kv) * dim:].float().view(n, n_kv // value_share, value_dim).repeat_interleave(value_share, dim=1)
         if q_weight is not None:
             q, k = self._rms(q, eps) * q_weight, self._rms(k, eps) * k_weight
         if cos_sin is not None:
@@ -469,9 +473,104 @@ class TorchOps(KernelNamespace):
         gate = torch.sigmoid(proj[:, gate_column:gate_column + heads].float()) if gate_column >= 0 else torch.ones(n, heads, device=y.device)
         out.copy_((y.float().transpose(0, 1) * gate[..., None]).reshape(n, heads * v).to(out.dtype))
 
+    # -- a block whose sublayers join the stream together; differential attention; the gated delta rule -----------------
+    def gated_pair_update(self, x, gates, y1, scale1, y2, scale2, next_weight=None, next_eps=0.0, normed=None):
+        width = x.shape[1]
+        g = torch.sigmoid(gates.float())
+        x += scale1 * g[:, :width] * y1.float()
+        if y2 is not None:
+            x += scale2 * g[:, width:] * y2.float()
+        if next_weight is not None:
+            normed.copy_((self._rms(x, next_eps) * next_weight).to(normed.dtype))
+
+    def differential_heads(self, attended, lam, keep, eps, out, kv_heads, group, value_dim, row):
+        n = attended.shape[0]
+        maps = attended.float().view(n, kv_heads, 2, group, row)[..., :value_dim]
+        d = maps[:, :, 0] - lam * maps[:, :, 1]
+        out.copy_((self._rms(d, eps) * keep).reshape(n, kv_heads * group * value_dim).to(out.dtype))
+
+    def delta_prepare(self, proj, taps, state, offset, state_slots, token_row, positions, row_start, out, kv_heads, heads, dim,
+                      value_dim, q_scale, unit_eps, keep=False):
+        channels, count = taps.shape
+        kept = count - 1
+        x = proj[:, :channels].float()
+        result = torch.zeros_like(x)
+        for t in range(x.shape[0]):
+            row, position = int(token_row[t]), int(positions[t])
+            first = position - (t - int(row_start[row]))
+            slot = int(state_slots[row])
+            old = state[slot, offset:offset + kept * channels].view(kept, channels)
+            for j in range(count):
+                back = kept - j
+                place = position - back
+                if place < 0:
+                    continue
+                value = x[t - back] if place >= first else old[kept - (first - place)]
+                result[t] += taps[:, j] * value
+        result = result * torch.sigmoid(result)
+        keys = kv_heads * dim
+        for start in (0, keys):
+            part = result[:, start:start + keys].view(-1, kv_heads, dim)
+            part = part / torch.sqrt(part.pow(2).sum(dim=-1, keepdim=True) + unit_eps)
+            result[:, start:start + keys] = (part * (q_scale if start == 0 else 1.0)).reshape(-1, keys)
+        out.copy_(result)
+        if keep and kept:
+            assert x.shape[0] == len(row_start)
+            for t in range(x.shape[0]):
+                slot = int(state_slots[int(token_row[t])])
+                old = state[slot, offset:offset + kept * channels].view(kept, channels)
+                state[slot, offset:offset + kept * channels] = torch.cat([old[1:], x[t:t + 1]], dim=0).reshape(-1)
+
+    def delta_conv_keep(self, proj, channels, taps, state, offset, state_slots, row_start, row_len, row_ctx):
+        kept = taps - 1
+        x = proj[:, :channels].float()
+        for row in range(len(row_len)):
+            slot, start, count, end = int(state_slots[row]), int(row_start[row]), int(row_len[row]), int(row_ctx[row])
+            if count <= 0:
+                continue
+            first = end - count
+            old = state[slot, offset:offset + kept * channels].view(kept, channels).clone()
+            new = torch.zeros_like(old)
+            for k in range(kept):
+                place = end - kept + k
+                if place >= first:
+                    new[k] = x[start + place - first]
+                elif place >= 0:
+                    new[k] = old[k + count]
+            state[slot, offset:offset + kept * channels] = new.reshape(-1)
+
+    def delta_rule(self, prepared, strength, decay, decay_scale, decay_bias, per_channel, state, offset, state_slots, row_start,
+                   row_len, row_ctx, out, heads, kv_heads, dim, value_dim):
+        keys, size, repeat = kv_heads * dim, heads * dim * value_dim, heads // kv_heads
+        beta = torch.sigmoid(strength.float())
+        step = torch.nn.functional.softplus(decay.float() + decay_bias)
+        if per_channel:
+            g = torch.exp(-torch.exp(decay_scale)[None, :, None] * step.view(-1, heads, dim))[..., None]
+        else:
+            g = torch.exp(-torch.exp(decay_scale) * step)[:, :, None, None]
+        for row in range(len(row_len)):
+            start, count, end = int(row_start[row]), int(row_len[row]), int(row_ctx[row])
+            if count <= 0:
+                continue
+            slot = int(state_slots[row])
+            matrix = state[slot, offset:offset + size].view(heads, dim, value_dim).clone()
+            if end - count == 0:
+                matrix.zero_()
+            for t in range(start, start + count):
+                q = prepared[t, :keys].view(kv_heads, dim).repeat_interleave(repeat, dim=0)
+                k = prepared[t, keys:2 * keys].view(kv_heads, dim).repeat_interleave(repeat, dim=0)
+                v = prepared[t, 2 * keys:].view(heads, value_dim)
+                matrix = matrix * g[t]
+                u = beta[t][:, None] * (v - torch.einsum("hdv,hd->hv", matrix, k))
+                matrix = matrix + k[:, :, None] * u[:, None, :]
+                out[t] = torch.einsum("hdv,hd->hv", matrix, q).reshape(-1)
+            state[slot, offset:offset + size] = matrix.reshape(-1)
+
     # -- routed experts ----------------------------------------------------------------------------------
-    def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None):
+    def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None, bias=None):
         logits = x.float() @ router.float().t()
+        if bias is not None:
+            logits = logits + bias
         if scoring == "softmax":
             best = torch.topk(logits, top, dim=-1)
             chosen.copy_(best.indices.to(chosen.dtype))
