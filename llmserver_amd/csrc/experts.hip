@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void route_logits_kernel(const float* __restri
 // each round with the same (best, where).
 __global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict__ all_logits, int experts, int top,
                                                         int* __restrict__ chosen, float* __restrict__ weights, int n_tokens,
-                                                        int sigmoid_scores, int groups, int keep) {
+                                                        int sigmoid_scores, int groups, int keep, const float* __restrict__ bias) {
     extern __shared__ float lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = blockIdx.x * (blockDim.x >> 6) + wave;
@@ -101,6 +101,7 @@ __global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict_
     float* scores = logits + experts;
     for (int e = lane; e < experts; e += 64) {
         float v = all_logits[(size_t)t * experts + e];
+        if (bias) v += bias[e];                            // (a bias per expert joins the logits)
         if (sigmoid_scores) v = 1.f / (1.f + expf(-v));
         logits[e] = v;
         scores[e] = v;
@@ -260,12 +261,12 @@ LSA_EXPORT int lsa_route_logits(const float* x, const float* router, float* logi
 // sigmoid_scores: the choice is made among sigmoid(logits), which are the weights as they are; groups > 1: only the
 // experts of the `keep` best of `groups` equal groups of neighbours can be chosen (at most 64 groups).
 LSA_EXPORT int lsa_route_top(const float* logits, int experts, int top, int* chosen, float* weights, int n, int sigmoid_scores,
-                             int groups, int keep, hipStream_t stream) {
+                             int groups, int keep, const float* bias, hipStream_t stream) {
     if (n <= 0) return 0;
     if (top < 1 || top > experts || (size_t)experts * 32 > 60000) return -1;
     if (groups > 1 && (!sigmoid_scores || groups > 64 || experts % groups || keep < 1 || keep > groups || top > keep * (experts / groups))) return -1;
     route_top_kernel<<<(n + 3) / 4, 256, (size_t)experts * 8 * sizeof(float), stream>>>(logits, experts, top, chosen, weights, n,
-                                                                                       sigmoid_scores, groups, keep);
+                                                                                       sigmoid_scores, groups, keep, bias);
     LSA_LAUNCH_CHECK();
 }
 

@@ -280,7 +280,7 @@ __global__ __launch_bounds__(64) void qkv_prepare_kernel(const T* __restrict__ q
                                                          const int* __restrict__ positions, const float* __restrict__ q_weight,
                                                          const float* __restrict__ k_weight, float eps, const float* __restrict__ cos_sin,
                                                          int pairs, int page_size, int n_q, int n_kv, int dim, int value_dim, int D,
-                                                         T* __restrict__ out_q, int write_cache, int halves) {
+                                                         T* __restrict__ out_q, int write_cache, int halves, int value_share) {
     const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const bool is_query = head < n_q;
     if (!is_query && !write_cache) return;
@@ -320,7 +320,8 @@ __global__ __launch_bounds__(64) void qkv_prepare_kernel(const T* __restrict__ q
     if (page < 0) return;
     T* key = keys + (((size_t)page * n_kv + kv) * page_size + slot) * D;
     T* value = values + ((size_t)page * n_kv + kv) * D * page_size + slot;
-    const T* v = qkv + (size_t)t * stride + (size_t)(n_q + n_kv) * dim + (size_t)kv * value_dim;
+    // (value_share neighbouring key heads read one value head: the projection has n_kv / value_share of them)
+    const T* v = qkv + (size_t)t * stride + (size_t)(n_q + n_kv) * dim + (size_t)(kv / value_share) * value_dim;
     for (int e = lane; e < D; e += 64) {
         key[e] = (T)prepared(e);
         value[(size_t)e * page_size] = e < value_dim ? v[e] : (T)0.f;
@@ -330,12 +331,13 @@ __global__ __launch_bounds__(64) void qkv_prepare_kernel(const T* __restrict__ q
 LSA_EXPORT int lsa_qkv_prepare(int dtype, const void* qkv, long stride, void* keys, void* values, const int* table, int table_stride,
                                const int* token_row, const int* positions, const float* q_weight, const float* k_weight, float eps,
                                const float* cos_sin, int pairs, int page_size, int n_q, int n_kv, int dim, int value_dim, int D,
-                               void* out_q, int write_cache, int n_tokens, int halves, hipStream_t stream) {
+                               void* out_q, int write_cache, int n_tokens, int halves, int value_share, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (value_share < 1 || n_kv % value_share) return -1;
     if (dim > D || value_dim > D || 2 * pairs > dim || page_size <= 0 || (q_weight == nullptr) != (k_weight == nullptr)) return -1;
     dim3 grid(n_tokens, n_q + n_kv);
 #define LSA_LAUNCH(T) qkv_prepare_kernel<T><<<grid, 64, 0, stream>>>((const T*)qkv, stride, (T*)keys, (T*)values, table, table_stride, token_row, \
-        positions, q_weight, k_weight, eps, cos_sin, pairs, page_size, n_q, n_kv, dim, value_dim, D, (T*)out_q, write_cache, halves)
+        positions, q_weight, k_weight, eps, cos_sin, pairs, page_size, n_q, n_kv, dim, value_dim, D, (T*)out_q, write_cache, halves, value_share)
     if (dtype) LSA_LAUNCH(bf16_t); else LSA_LAUNCH(float);
 #undef LSA_LAUNCH
     LSA_LAUNCH_CHECK();

@@ -27,8 +27,8 @@ FLAGS = ["-O3", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-std=c++17",
 HEAD_DIMS = tuple(range(16, 257, 16))
 BASE_MODULES = ("elementwise", "rope_kv", "sampling", "gemm")
 # Libraries that only some models call (a 32-bit residual stream, attention over a latent, routed experts, mixers with a
-# recurrent state): loaded, and compiled if need be, when the first such call is made.
-PART_MODULES = ("stream", "latent", "experts", "recurrent")
+# recurrent state, the delta rule): loaded, and compiled if need be, when the first such call is made.
+PART_MODULES = ("stream", "latent", "experts", "recurrent", "delta")
 
 
 class KernelBuildError(RuntimeError):

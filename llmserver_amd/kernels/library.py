@@ -34,7 +34,7 @@ _SIGNATURES = {
                           c_int, c_int, c_int, c_int, _P, _P, c_int, _P],
     "lsa_norm_add_norm": [_P, _P, _P, c_int, c_float, c_float, _P, c_float, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_qkv_prepare": [c_int, _P, c_long, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                        _P, c_int, c_int, c_int, _P],
+                        _P, c_int, c_int, c_int, c_int, _P],
     "lsa_token_shift": [c_int, _P, _P, c_int, _P, c_long, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P],
     "lsa_token_shift_keep": [c_int, _P, _P, c_long, _P, _P, _P, c_int, c_int, _P],
     "lsa_linear_recurrence_most_dim": [],
@@ -53,7 +53,14 @@ _SIGNATURES = {
                            c_int, c_int, c_int, c_int, _P],
     "lsa_gate_heads": [c_int, _P, _P, _P, c_int, c_int, _P, c_long, c_int, _P, c_int, c_int, c_int, c_int, _P],
     "lsa_route_logits": [_P, _P, _P, c_int, c_int, c_int, _P],
-    "lsa_route_top": [_P, c_int, c_int, _P, _P, c_int, c_int, c_int, c_int, _P],
+    "lsa_route_top": [_P, c_int, c_int, _P, _P, c_int, c_int, c_int, c_int, _P, _P],
+    "lsa_gated_pair_update": [_P, _P, c_int, c_int, _P, c_int, _P, _P, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
+    "lsa_differential_heads": [c_int, _P, c_float, c_float, c_float, _P, c_int, c_int, c_int, c_int, c_int, _P],
+    "lsa_delta_most_dim": [],
+    "lsa_delta_prepare": [c_int, _P, c_long, _P, c_int, _P, c_long, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
+                          _P, c_long, _P, c_long, c_int, _P, _P, _P, _P, c_int, _P],
+    "lsa_delta_conv_keep": [c_int, _P, c_long, _P, c_long, _P, _P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_delta_rule": [_P, _P, _P, c_int, _P, c_long, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
     "lsa_experts_gate_up": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P],
     "lsa_experts_tile_rows": [],
     "lsa_experts_tiled": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P],

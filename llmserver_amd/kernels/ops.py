@@ -1006,14 +1006,17 @@ class HipOps(KernelNamespace):
                                                               proj.shape[1], int(gate_column), _ptr(out), heads, v, n, 1 if per_channel else 0,
                                                               _stream()), "gate_heads")
 
-    def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None):
-        """The logits are a float32 product of the library (no reduced-precision mode), the choice and the weights a kernel."""
+    def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None, bias=None):
+        """The logits are a float32 product of the library (no reduced-precision mode), the choice and the weights a kernel
+        (which also adds the bias)."""
         n, width = x.shape
         experts = router.shape[0]
         _check(x, "x")
         _check(router, "router", torch.float32, (experts, width))
         _check(chosen, "chosen", torch.int32, (n, top))
         _check(weights, "weights", torch.float32, (n, top))
+        if bias is not None:
+            _check(bias, "bias", torch.float32, (experts,))
         if not 1 <= top <= experts or experts > 3072:
             raise ValueError(f"the router kernel chooses 1 to {min(experts, 3072)} of up to 3072 experts, asked for {top} of {experts}")
         wide = x if x.dtype == torch.float32 else x.float()
@@ -1029,7 +1032,8 @@ class HipOps(KernelNamespace):
         if count > 64 or experts % count or not 1 <= keep <= count or top > keep * (experts // count):
             raise ValueError(f"the router kernel takes up to 64 equal groups: {experts} experts in {count} groups, {keep} kept, {top} chosen")
         _launched(self._part_library("experts").lsa_route_top(_ptr(logits), experts, top, _ptr(chosen), _ptr(weights), n,
-                                                              1 if scoring == "sigmoid" else 0, int(count), int(keep), _stream()), "route_top")
+                                                              1 if scoring == "sigmoid" else 0, int(count), int(keep), _ptr(bias), _stream()),
+                  "route_top")
 
     @staticmethod
     def _expert_limit(activation, limit) -> float:
@@ -1088,11 +1092,18 @@ class HipOps(KernelNamespace):
 
     # -- general preparation of queries, keys and values; mixers with a recurrent state -----------------------------
     def qkv_prepare(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
-                    n_q, n_kv, dim, value_dim, out_q, write_cache=True, pairing="neighbours"):
+                    n_q, n_kv, dim, value_dim, out_q, write_cache=True, pairing="neighbours", value_share=1):
+        """``value_share``: so many neighbouring key heads read one value head (``qkv`` brings ``n_kv / value_share`` of them).
+        Without ``write_cache`` only the queries are read, and ``qkv`` may bring nothing else."""
         n = qkv.shape[0]
         if pairing not in ("neighbours", "halves"):
             raise ValueError(f"dimensions turn in neighbouring pairs or in halves, not {pairing!r}")
-        _check(qkv, "qkv", None, (n, (n_q + n_kv) * dim + n_kv * value_dim))
+        if value_share < 1 or n_kv % value_share:
+            raise ValueError(f"{n_kv} key heads do not share values in groups of {value_share}")
+        if write_cache or qkv.shape[1] != n_q * dim:
+            _check(qkv, "qkv", None, (n, (n_q + n_kv) * dim + (n_kv // value_share) * value_dim))
+        else:
+            _check(qkv, "qkv", None, (n, n_q * dim))
         pages, row = keys.shape[0], keys.shape[-1]
         _check(keys, "keys", qkv.dtype, (pages, n_kv, page_size, row))
         _check(values, "values", qkv.dtype, (pages, n_kv, row, page_size))
@@ -1116,7 +1127,103 @@ class HipOps(KernelNamespace):
         _launched(self._rope_kv.lsa_qkv_prepare(
             _code(qkv), _ptr(qkv), qkv.shape[1], _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(token_row), _ptr(positions),
             _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin), pairs, page_size, n_q, n_kv, dim, value_dim, row, _ptr(out_q),
-            1 if write_cache else 0, n, 1 if pairing == "halves" else 0, _stream()), "qkv_prepare")
+            1 if write_cache else 0, n, 1 if pairing == "halves" else 0, int(value_share), _stream()), "qkv_prepare")
+
+    # -- a block whose sublayers join the stream together; differential attention; the gated delta rule ------------------
+    def gated_pair_update(self, x, gates, y1, scale1, y2, scale2, next_weight=None, next_eps=0.0, normed=None):
+        n, width = x.shape
+        _check(x, "x", torch.float32)
+        _check(gates, "gates", None, (n, 2 * width if y2 is not None else width))
+        _check(y1, "y1", None, (n, width))
+        _check(scale1, "scale1", torch.float32, (width,))
+        if y2 is not None:
+            _check(y2, "y2", None, (n, width))
+            _check(scale2, "scale2", torch.float32, (width,))
+        if next_weight is not None:
+            _check(next_weight, "next_weight", torch.float32, (width,))
+            _check(normed, "normed", None, (n, width))
+        _launched(self._part_library("delta").lsa_gated_pair_update(
+            _ptr(x), _ptr(gates), _code(gates), gates.shape[1], _ptr(y1), _code(y1), _ptr(scale1), _ptr(y2), _code(y2) if y2 is not None else 0,
+            _ptr(scale2) if y2 is not None else None, _ptr(next_weight), float(next_eps), _ptr(normed) if next_weight is not None else None,
+            _code(normed) if next_weight is not None else 0, n, width, _stream()), "gated_pair_update")
+
+    def differential_heads(self, attended, lam, keep, eps, out, kv_heads, group, value_dim, row):
+        n = attended.shape[0]
+        _check(attended, "attended", None, (n, kv_heads * 2 * group * row))
+        _check(out, "out", attended.dtype, (n, kv_heads * group * value_dim))
+        _launched(self._part_library("delta").lsa_differential_heads(_code(attended), _ptr(attended), float(lam), float(keep), float(eps), _ptr(out),
+                                                                     n, kv_heads, group, value_dim, row, _stream()), "differential_heads")
+
+    @staticmethod
+    def _strided(tensor, name, rows, columns, dtype=None):
+        if not tensor.is_cuda or (dtype is not None and tensor.dtype != dtype) or tuple(tensor.shape) != (rows, columns) \
+                or (columns > 1 and tensor.stride(1) != 1):
+            raise ValueError(f"{name} must be a view [{rows}, {columns}] of {dtype} on the GPU with unit stride along a row")
+
+    def delta_prepare(self, proj, taps, state, offset, state_slots, token_row, positions, row_start, out, kv_heads, heads, dim,
+                      value_dim, q_scale, unit_eps, strength, decay, decay_scale, decay_bias, per_channel, out_strength, out_decay,
+                      keep=False):
+        n = proj.shape[0]
+        channels, count = taps.shape
+        rows = row_start.shape[0]
+        if keep and n != rows:
+            raise ValueError("the state moves on inside this kernel only in steps of one token per row")
+        lib = self._part_library("delta")
+        if channels != 2 * kv_heads * dim + heads * value_dim or dim > lib.lsa_delta_most_dim():
+            raise ValueError(f"{channels} channels for {kv_heads} key heads of {dim} (up to {lib.lsa_delta_most_dim()}) and {heads} value heads of {value_dim}")
+        if not proj.is_cuda or proj.dim() != 2 or proj.shape[1] < channels or proj.stride(1) != 1:
+            raise ValueError(f"proj must bring at least {channels} columns with unit stride along a row")
+        _code(proj)
+        _check(taps, "taps", torch.float32)
+        _check(out, "out", torch.float32, (n, channels))
+        _check(token_row, "token_row", torch.int32, (n,))
+        _check(positions, "positions", torch.int32, (n,))
+        _check(row_start, "row_start", torch.int32)
+        _check(state_slots, "state_slots", torch.int32, (rows,))
+        self._strided(strength, "strength", n, heads, proj.dtype)
+        if per_channel:
+            _check(decay, "decay", torch.float32, (n, heads * dim))
+        else:
+            self._strided(decay, "decay", n, heads, proj.dtype)
+        _check(decay_scale, "decay_scale", torch.float32, (heads,))
+        _check(decay_bias, "decay_bias", torch.float32, (heads * dim if per_channel else heads,))
+        _check(out_strength, "out_strength", torch.float32, (n, heads))
+        _check(out_decay, "out_decay", torch.float32, (n, heads * dim if per_channel else heads))
+        pointer, stride = self._state_rows(state, offset, (count - 1) * channels, "state")
+        _launched(lib.lsa_delta_prepare(
+            _code(proj), proj.data_ptr(), proj.stride(0), _ptr(taps), count, pointer, stride, _ptr(state_slots), _ptr(token_row), _ptr(positions),
+            _ptr(row_start), _ptr(out), kv_heads, heads, dim, value_dim, float(q_scale), float(unit_eps), 1 if keep else 0,
+            strength.data_ptr(), strength.stride(0), decay.data_ptr(), decay.stride(0), 1 if per_channel else 0, _ptr(decay_scale),
+            _ptr(decay_bias), _ptr(out_strength), _ptr(out_decay), n, _stream()), "delta_prepare")
+
+    def delta_conv_keep(self, proj, channels, taps, state, offset, state_slots, row_start, row_len, row_ctx):
+        rows = row_len.shape[0]
+        if not proj.is_cuda or proj.dim() != 2 or proj.shape[1] < channels or proj.stride(1) != 1:
+            raise ValueError(f"proj must bring at least {channels} columns with unit stride along a row")
+        for name, tensor in (("state_slots", state_slots), ("row_start", row_start), ("row_len", row_len), ("row_ctx", row_ctx)):
+            _check(tensor, name, torch.int32, (rows,))
+        pointer, stride = self._state_rows(state, offset, (taps - 1) * channels, "state")
+        _launched(self._part_library("delta").lsa_delta_conv_keep(_code(proj), proj.data_ptr(), proj.stride(0), pointer, stride, _ptr(state_slots),
+                                                                  _ptr(row_start), _ptr(row_len), _ptr(row_ctx), taps - 1, channels, rows, _stream()),
+                  "delta_conv_keep")
+
+    def delta_rule(self, prepared, strength, decay, per_channel, state, offset, state_slots, row_start, row_len, row_ctx, out,
+                   heads, kv_heads, dim, value_dim):
+        n = out.shape[0]
+        rows = row_len.shape[0]
+        lib = self._part_library("delta")
+        if dim > lib.lsa_delta_most_dim() or heads % kv_heads:
+            raise ValueError(f"the delta kernel takes heads of up to {lib.lsa_delta_most_dim()} key channels in whole groups, got {dim}, {heads}/{kv_heads}")
+        _check(prepared, "prepared", torch.float32, (n, 2 * kv_heads * dim + heads * value_dim))
+        _check(strength, "strength", torch.float32, (n, heads))
+        _check(decay, "decay", torch.float32, (n, heads * dim if per_channel else heads))
+        _check(out, "out", torch.float32, (n, heads * value_dim))
+        for name, tensor in (("state_slots", state_slots), ("row_start", row_start), ("row_len", row_len), ("row_ctx", row_ctx)):
+            _check(tensor, name, torch.int32, (rows,))
+        pointer, stride = self._state_rows(state, offset, heads * dim * value_dim, "state")
+        _launched(lib.lsa_delta_rule(_ptr(prepared), _ptr(strength), _ptr(decay), 1 if per_channel else 0, pointer, stride, _ptr(state_slots),
+                                     _ptr(row_start), _ptr(row_len), _ptr(row_ctx), _ptr(out), rows, heads, kv_heads, dim, value_dim, _stream()),
+                  "delta_rule")
 
     @staticmethod
     def _state_rows(state, offset, needed, name):

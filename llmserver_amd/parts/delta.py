@@ -168,14 +168,17 @@ class GatedDeltaRule(Mixer):
             gate = self.gate_up.forward(gate.contiguous(), ctx)
         single = ctx.n_tokens == ctx.n_rows         # one token a row: the workgroup that reads a row's last inputs also moves them on
         prepared = ctx.empty((n, self.channels), dtype=torch.float32)
+        strengths = ctx.empty((n, self.heads), dtype=torch.float32)
+        decays = ctx.empty((n, self.heads * self.dim if self.decay_per_channel else self.heads), dtype=torch.float32)
         ops.delta_prepare(proj, self.conv_weight, cache.state, self.matrix_size, ctx.state_slots, ctx.token_row, ctx.positions,
-                          ctx.row_start, prepared, self.kv_heads, self.heads, self.dim, self.value_dim, self.q_scale, UNIT_EPS, keep=single)
+                          ctx.row_start, prepared, self.kv_heads, self.heads, self.dim, self.value_dim, self.q_scale, UNIT_EPS,
+                          strength, decay, self.decay_scale, self.decay_bias, self.decay_per_channel, strengths, decays, keep=single)
         if not single and self.taps > 1:
             ops.delta_conv_keep(proj, self.channels, self.taps, cache.state, self.matrix_size, ctx.state_slots, ctx.row_start,
                                 ctx.row_len, ctx.row_ctx)
         mixed = ctx.empty((n, self.values), dtype=torch.float32)
-        ops.delta_rule(prepared, strength, decay, self.decay_scale, self.decay_bias, self.decay_per_channel, cache.state, 0,
-                       ctx.state_slots, ctx.row_start, ctx.row_len, ctx.row_ctx, mixed, self.heads, self.kv_heads, self.dim, self.value_dim)
+        ops.delta_rule(prepared, strengths, decays, self.decay_per_channel, cache.state, 0, ctx.state_slots, ctx.row_start, ctx.row_len,
+                       ctx.row_ctx, mixed, self.heads, self.kv_heads, self.dim, self.value_dim)
         gated = ctx.empty((n, self.values))
         ops.heads_norm_gate(mixed, self.norm_weight, False, self.norm_eps, gate, gated, self.heads, self.value_dim,
                             gate_activation="sigmoid" if self.low_rank_gate else "silu")

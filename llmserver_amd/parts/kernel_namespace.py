@@ -212,13 +212,16 @@ class KernelNamespace:
 
     # The gated delta rule.
     def delta_prepare(self, proj, taps, state, offset, state_slots, token_row, positions, row_start, out, kv_heads, heads, dim,
-                      value_dim, q_scale, unit_eps, keep=False):
+                      value_dim, q_scale, unit_eps, strength, decay, decay_scale, decay_bias, per_channel, out_strength, out_decay,
+                      keep=False):
         """The first ``C = 2 * kv_heads * dim + heads * value_dim`` columns of ``proj`` (queries, keys, values) pass a causal
         convolution over each request's tokens per channel (``taps [C, K]``, tap ``j`` on the token ``K - 1 - j`` places
         back, zeros before the sequence, earlier steps' inputs from ``state[slot, offset:]`` as ``[K - 1, C]``, oldest first)
         and silu; every query and key head is then divided by ``sqrt(sum of its squares + unit_eps)``, queries also times
-        ``q_scale``.  ``out [T, C]`` float32.  ``keep`` (steps of one token per row only): the state also moves on by the
-        step's token, as :meth:`delta_conv_keep` would do."""
+        ``q_scale``.  ``out [T, C]`` float32.  Beside them ``out_strength [T, heads] = sigmoid(strength)`` and
+        ``out_decay = exp(-exp(decay_scale[h]) * softplus(decay + decay_bias))`` with ``decay [T, heads]`` and ``decay_bias
+        [heads]``, or, ``per_channel``, ``decay [T, heads * dim]`` float32 and ``decay_bias [heads * dim]``.  ``keep`` (steps of
+        one token per row only): the state also moves on by the step's token, as :meth:`delta_conv_keep` would do."""
         raise NotImplementedError
 
     def delta_conv_keep(self, proj, channels, taps, state, offset, state_slots, row_start, row_len, row_ctx):
@@ -226,14 +229,13 @@ class KernelNamespace:
         fewer) into ``state[slot, offset:]``."""
         raise NotImplementedError
 
-    def delta_rule(self, prepared, strength, decay, decay_scale, decay_bias, per_channel, state, offset, state_slots, row_start,
-                   row_len, row_ctx, out, heads, kv_heads, dim, value_dim):
+    def delta_rule(self, prepared, strength, decay, per_channel, state, offset, state_slots, row_start, row_len, row_ctx, out,
+                   heads, kv_heads, dim, value_dim):
         """Per head ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` over each row's tokens, with
-        ``prepared [T, C]`` from :meth:`delta_prepare` (head ``h`` reads query/key head ``h // (heads / kv_heads)``),
-        ``beta = sigmoid(strength[t, h])``, ``g = exp(-exp(decay_scale[h]) * softplus(decay + decay_bias))`` with ``decay [T,
-        heads]`` and ``decay_bias [heads]``, or, ``per_channel``, ``decay [T, heads * dim]`` float32 and ``decay_bias [heads *
-        dim]``: a decay for every row of ``S``.  ``S [heads, dim, value_dim]`` float32 lives in ``state[slot, offset:]``, zeros
-        before a sequence's first token.  ``out [T, heads * value_dim]`` float32."""
+        ``prepared [T, C]``, ``strength [T, heads]`` (beta) and ``decay`` (g: ``[T, heads]``, or, ``per_channel``, ``[T, heads *
+        dim]``, a decay for every row of ``S``) from :meth:`delta_prepare`; head ``h`` reads query/key head ``h // (heads /
+        kv_heads)``.  ``S [heads, dim, value_dim]`` float32 lives in ``state[slot, offset:]``, zeros before a sequence's first
+        token.  ``out [T, heads * value_dim]`` float32."""
         raise NotImplementedError
 
     # Routed experts.

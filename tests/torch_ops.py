@@ -490,7 +490,12 @@ class TorchOps(KernelNamespace):
         out.copy_((self._rms(d, eps) * keep).reshape(n, kv_heads * group * value_dim).to(out.dtype))
 
     def delta_prepare(self, proj, taps, state, offset, state_slots, token_row, positions, row_start, out, kv_heads, heads, dim,
-                      value_dim, q_scale, unit_eps, keep=False):
+                      value_dim, q_scale, unit_eps, strength, decay, decay_scale, decay_bias, per_channel, out_strength, out_decay,
+                      keep=False):
+        out_strength.copy_(torch.sigmoid(strength.float()))
+        step = torch.nn.functional.softplus(decay.float() + decay_bias)
+        rate = torch.exp(decay_scale)
+        out_decay.copy_(torch.exp(-(rate[None, :, None] * step.view(-1, heads, dim)).reshape(step.shape[0], -1) if per_channel else -rate * step))
         channels, count = taps.shape
         kept = count - 1
         x = proj[:, :channels].float()
@@ -539,15 +544,11 @@ class TorchOps(KernelNamespace):
                     new[k] = old[k + count]
             state[slot, offset:offset + kept * channels] = new.reshape(-1)
 
-    def delta_rule(self, prepared, strength, decay, decay_scale, decay_bias, per_channel, state, offset, state_slots, row_start,
-                   row_len, row_ctx, out, heads, kv_heads, dim, value_dim):
+    def delta_rule(self, prepared, strength, decay, per_channel, state, offset, state_slots, row_start, row_len, row_ctx, out,
+                   heads, kv_heads, dim, value_dim):
         keys, size, repeat = kv_heads * dim, heads * dim * value_dim, heads // kv_heads
-        beta = torch.sigmoid(strength.float())
-        step = torch.nn.functional.softplus(decay.float() + decay_bias)
-        if per_channel:
-            g = torch.exp(-torch.exp(decay_scale)[None, :, None] * step.view(-1, heads, dim))[..., None]
-        else:
-            g = torch.exp(-torch.exp(decay_scale) * step)[:, :, None, None]
+        beta = strength
+        g = decay.view(-1, heads, dim)[..., None] if per_channel else decay[:, :, None, None]
         for row in range(len(row_len)):
             start, count, end = int(row_start[row]), int(row_len[row]), int(row_ctx[row])
             if count <= 0:
