@@ -215,3 +215,12 @@ def forward(config, tensors, tokens, r=same, layer_outputs=None):
             layer_outputs.append(x.clone())
     final = r(scalar_norm(x, tensors["final.norm"], eps))
     return (final @ tensors["head"].T).to(dtype)
+
+
+def greedy_generate(config, tensors, prompt, count):
+    """The prompt's ``count`` most likely continuations, one token at a time, the first of equal logits."""
+    tokens, made = list(prompt), []
+    for _ in range(count):
+        made.append(int(torch.argmax(forward(config, tensors, tokens)[-1])))
+        tokens.append(made[-1])
+    return made
