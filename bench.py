@@ -197,7 +197,7 @@ def main() -> int:
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points")
     parser.add_argument("--no-extra-points", action="store_true", help="skip the Qwen3-1.7B-sized mixed workload and the Qwen3-32B-sized batch")
     parser.add_argument("--no-prefill", action="store_true")
-    parser.add_argument("--design", default="", choices=("", "zepolix", "barotar", "kerudra"),
+    parser.add_argument("--design", default="", choices=("", "zepolix", "barotar", "kerudra", "gogalix"),
                         help="instead of the default workload: prefill and decode of this design at a few named sizes, each beside "
                              "the dense decoder of equal width, depth and active feed-forward size")
     args = parser.parse_args()
@@ -295,7 +295,9 @@ UNMEASURED_DESIGNS = {}
 
 DESIGN_SIZES = {"zepolix": (("zepolix-2k", "dense-2k"), ("zepolix-4k", "dense-4k")),
                 "barotar": (("barotar-2k", "dense-2k"), ("barotar-4k", "dense-4k")),
-                "kerudra": (("kerudra-2k", "dense-2k"), ("kerudra-4k", "dense-4k"))}
+                "kerudra": (("kerudra-2k", "dense-2k"), ("kerudra-4k", "dense-4k")),
+                # (beside the dense decoder and beside the design whose layers are most like its own: recurrences, windows, experts)
+                "gogalix": (("gogalix-2k", "barotar-2k", "dense-2k"), ("gogalix-4k", "barotar-4k", "dense-4k"))}
 
 
 def compare_design(args) -> int:

@@ -99,6 +99,37 @@ NAMED_SIZES.update({
 })
 
 
+def _gogalix(width, layers, heads, kv_heads, dim, vdim, window, delta_heads, delta_kv_heads, delta_dim, delta_vdim, ff, expert_ff, experts, top,
+             vocab=32768):
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "diff": 0.6, "mask": {"size": window}}
+    delta = {"heads": delta_heads, "kv_heads": delta_kv_heads, "dim": delta_dim, "vdim": delta_vdim, "conv": 4}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}}
+    made = []
+    for index in range(layers):
+        kind = index % 4
+        if kind == 0:
+            made.append({"type": "attention", "mixer": dict(attention), "mlp": dict(dense)})
+        elif kind == 1:
+            made.append({"type": "delta", "mixer": dict(delta), "mlp": dict(moe)})
+        elif kind == 2:
+            made.append({"type": "channel_delta", "mixer": {**delta, "low": 64, "gate_low": 64}, "mlp": dict(dense)})
+        else:
+            made.append({"type": "attention", "mixer": {**attention, "kv_from": index - 3}, "mlp": dict(moe)})
+    return {"architecture": "Gogalix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0}, "layers": made}
+
+
+# Gogalix at the widths of the sizes above: of every four layers one is differential attention of 16 (32) heads with two maps
+# of 64 and values of 128 over 8 key/value heads under a window of 1,024 keys, one reads that layer's pages with queries of
+# its own, and two are gated delta rules of 16 (32) heads with keys and values of 128 over 8 (16) key heads (a state of 1 MB
+# (2 MB) a layer and request), one with a decay per head and one with a decay per key channel; dense feed-forwards as large
+# as the dense decoders' beside them in two layers of four, experts of the Zepolix sizes' shape in the other two.
+NAMED_SIZES.update({
+    "gogalix-2k": _gogalix(2048, 8, 16, 8, 64, 128, 1024, 16, 8, 128, 128, 6 * 1408, 1408, 64, 6),
+    "gogalix-4k": _gogalix(4096, 8, 32, 8, 64, 128, 1024, 32, 16, 128, 128, 4 * 2048, 2048, 32, 4),
+})
+
+
 def named_size(name: str) -> dict:
     """The entry's keys, a copy the caller may change (fewer layers, say)."""
     try:
