@@ -183,6 +183,30 @@ __device__ inline float sum_of_16(float v) {
     return v;
 }
 
+// One token of a column's walk: `S` the lane's key channels of the column, `kp`, `qp`, `gp` the token's key, query and
+// decays as the lane's part reads them, `g` the head's decay where there is one a head.
+template <int DP, bool PER_CHANNEL>
+__device__ inline float delta_token(float (&S)[DP], const float* __restrict__ kp, const float* __restrict__ qp, const float* __restrict__ gp,
+                                    float g, float beta, float v) {
+    float k[DP], seen[2] = {0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < DP; ++i) {
+        k[i] = kp[i];
+        S[i] *= PER_CHANNEL ? gp[i] : g;
+        seen[i & 1] += S[i] * k[i];
+    }
+    const float u = beta * (v - sum_of_16(seen[0] + seen[1]));
+    float read[2] = {0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < DP; ++i) {
+        S[i] += k[i] * u;
+        read[i & 1] += S[i] * qp[i];
+    }
+    return sum_of_16(read[0] + read[1]);
+}
+
+// state[slot]: per head and block of 16 value columns a tile [dim][16], so that a workgroup's share of the state is one
+// contiguous piece, read and written 16 bytes a thread and turned into the lanes' order through LDS.
 template <int DP, bool PER_CHANNEL>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ prepared, const float* __restrict__ strength,
                                                          const float* __restrict__ decay, float* state, long state_stride,
@@ -190,6 +214,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                                                          const int* __restrict__ row_len, const int* __restrict__ row_ctx,
                                                          float* __restrict__ out, int heads, int kv_heads, int dim, int value_dim) {
     constexpr int PADDED = DP * PARTS;
+    static_assert(CHUNK == BLOCK_COLUMNS, "the staging buffer of the queries doubles as the state's tile");
     __shared__ __align__(16) float s_q[CHUNK][PADDED], s_k[CHUNK][PADDED], s_g[PER_CHANNEL ? CHUNK : 1][PER_CHANNEL ? PADDED : 1];
     __shared__ float s_v[CHUNK][BLOCK_COLUMNS], s_beta[CHUNK], s_decay[CHUNK];
     const int row = blockIdx.x, head = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -198,16 +223,26 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
     const int start = row_start[row];
     const bool fresh = row_ctx[row] - count == 0;
     const int p = lane & (PARTS - 1);
-    const int column = blockIdx.z * BLOCK_COLUMNS + wave * 4 + (lane >> 4);
+    const int local = wave * 4 + (lane >> 4);
+    const int column = blockIdx.z * BLOCK_COLUMNS + local;
     const bool live = column < value_dim;
     const int kv_head = head / (heads / kv_heads);
     const int keys = kv_heads * dim, channels = 2 * keys + heads * value_dim;
-    float* matrix = state + (size_t)slots[row] * state_stride + (size_t)head * dim * value_dim;
+    float* tile = state + (size_t)slots[row] * state_stride + ((size_t)head * gridDim.z + blockIdx.z) * dim * BLOCK_COLUMNS;
+    float* turned = &s_q[0][0];                     // [PADDED][16], rows beyond dim unused
     float S[DP];
+    if (fresh) {
 #pragma unroll
-    for (int i = 0; i < DP; ++i) {
-        const int ch = i * PARTS + p;
-        S[i] = (!fresh && live && ch < dim) ? matrix[(size_t)ch * value_dim + column] : 0.f;
+        for (int i = 0; i < DP; ++i) S[i] = 0.f;
+    } else {
+        for (int piece = tid; piece < dim * (BLOCK_COLUMNS / 4); piece += 256)
+            reinterpret_cast<float4*>(turned)[piece] = reinterpret_cast<const float4*>(tile)[piece];
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < DP; ++i) {
+            const int ch = i * PARTS + p;
+            S[i] = (ch < dim && live) ? turned[ch * BLOCK_COLUMNS + local] : 0.f;      // (columns beyond the values stay zero)
+        }
     }
     for (int begin = 0; begin < count; begin += CHUNK) {
         const int tokens = min(CHUNK, count - begin);
@@ -232,45 +267,34 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
             if (!PER_CHANNEL) s_decay[tid] = decay[(size_t)(start + begin + tid) * heads + head];
         }
         __syncthreads();
-        for (int j = 0; j < tokens; ++j) {
-            const float* kp = &s_k[j][p * DP];
-            const float* qp = &s_q[j][p * DP];
-            float k[DP], seen[2] = {0.f, 0.f};
-            if (PER_CHANNEL) {
-                const float* gp = &s_g[j][p * DP];
+        float* o = out + (size_t)(start + begin) * heads * value_dim + (size_t)head * value_dim + column;
+        const bool writes = p == 0 && live;
+        if (tokens == CHUNK) {
+            // a whole chunk runs unrolled: a token's LDS loads are issued ahead of the token before it, and its read-out's
+            // sum across lanes overlaps the next token's walk
 #pragma unroll
-                for (int i = 0; i < DP; ++i) {
-                    k[i] = kp[i];
-                    S[i] *= gp[i];
-                    seen[i & 1] += S[i] * k[i];
-                }
-            } else {
-                const float g = s_decay[j];
-#pragma unroll
-                for (int i = 0; i < DP; ++i) {
-                    k[i] = kp[i];
-                    S[i] *= g;
-                    seen[i & 1] += S[i] * k[i];
-                }
+            for (int j = 0; j < CHUNK; ++j) {
+                const float r = delta_token<DP, PER_CHANNEL>(S, &s_k[j][p * DP], &s_q[j][p * DP], PER_CHANNEL ? &s_g[j][p * DP] : nullptr,
+                                                             PER_CHANNEL ? 1.f : s_decay[j], s_beta[j], s_v[j][local]);
+                if (writes) o[(size_t)j * heads * value_dim] = r;
             }
-            const float u = s_beta[j] * (s_v[j][wave * 4 + (lane >> 4)] - sum_of_16(seen[0] + seen[1]));
-            float read[2] = {0.f, 0.f};
-#pragma unroll
-            for (int i = 0; i < DP; ++i) {
-                S[i] += k[i] * u;
-                read[i & 1] += S[i] * qp[i];
+        } else {
+            for (int j = 0; j < tokens; ++j) {
+                const float r = delta_token<DP, PER_CHANNEL>(S, &s_k[j][p * DP], &s_q[j][p * DP], PER_CHANNEL ? &s_g[j][p * DP] : nullptr,
+                                                             PER_CHANNEL ? 1.f : s_decay[j], s_beta[j], s_v[j][local]);
+                if (writes) o[(size_t)j * heads * value_dim] = r;
             }
-            const float o = sum_of_16(read[0] + read[1]);
-            if (p == 0 && live) out[(size_t)(start + begin + j) * heads * value_dim + (size_t)head * value_dim + column] = o;
         }
     }
-    if (live) {
+    __syncthreads();
 #pragma unroll
-        for (int i = 0; i < DP; ++i) {
-            const int ch = i * PARTS + p;
-            if (ch < dim) matrix[(size_t)ch * value_dim + column] = S[i];
-        }
+    for (int i = 0; i < DP; ++i) {
+        const int ch = i * PARTS + p;
+        if (ch < dim) turned[ch * BLOCK_COLUMNS + local] = S[i];
     }
+    __syncthreads();
+    for (int piece = tid; piece < dim * (BLOCK_COLUMNS / 4); piece += 256)
+        reinterpret_cast<float4*>(tile)[piece] = reinterpret_cast<const float4*>(turned)[piece];
 }
 
 }  // namespace
@@ -304,6 +328,7 @@ LSA_EXPORT int lsa_differential_heads(int code, const void* attended, float lam,
 }
 
 LSA_EXPORT int lsa_delta_most_dim() { return MOST_DIM; }
+LSA_EXPORT int lsa_delta_state_columns() { return BLOCK_COLUMNS; }
 
 LSA_EXPORT int lsa_delta_prepare(int code, const void* proj, long stride, const float* w, int taps, float* state, long state_stride,
                                  const int* slots, const int* token_row, const int* positions, const int* row_start, float* out,
@@ -337,8 +362,8 @@ LSA_EXPORT int lsa_delta_rule(const float* prepared, const float* strength, cons
                               float* out, int rows, int heads, int kv_heads, int dim, int value_dim, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (dim < 1 || dim > MOST_DIM || heads < 1 || kv_heads < 1 || heads % kv_heads || value_dim < 1 || !state) return -1;
-    if (state_stride < (long)heads * dim * value_dim) return -1;
     dim3 grid(rows, heads, (value_dim + BLOCK_COLUMNS - 1) / BLOCK_COLUMNS);
+    if (state_stride < (long)heads * grid.z * dim * BLOCK_COLUMNS || state_stride % 4 || ((size_t)state % 16)) return -1;
     const int parts = (dim + PARTS - 1) / PARTS;
 #define LSA_LAUNCH(DP, PC) delta_rule_kernel<DP, PC><<<grid, 256, 0, stream>>>(prepared, strength, decay, state, state_stride, slots, row_start, \
         row_len, row_ctx, out, heads, kv_heads, dim, value_dim)

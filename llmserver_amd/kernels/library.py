@@ -57,6 +57,7 @@ _SIGNATURES = {
     "lsa_gated_pair_update": [_P, _P, c_int, c_int, _P, c_int, _P, _P, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_differential_heads": [c_int, _P, c_float, c_float, c_float, _P, c_int, c_int, c_int, c_int, c_int, _P],
     "lsa_delta_most_dim": [],
+    "lsa_delta_state_columns": [],
     "lsa_delta_prepare": [c_int, _P, c_long, _P, c_int, _P, c_long, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                           _P, c_long, _P, c_long, c_int, _P, _P, _P, _P, c_int, _P],
     "lsa_delta_conv_keep": [c_int, _P, c_long, _P, c_long, _P, _P, _P, _P, c_int, c_int, c_int, _P],

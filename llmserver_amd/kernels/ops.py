@@ -1220,7 +1220,10 @@ class HipOps(KernelNamespace):
         _check(out, "out", torch.float32, (n, heads * value_dim))
         for name, tensor in (("state_slots", state_slots), ("row_start", row_start), ("row_len", row_len), ("row_ctx", row_ctx)):
             _check(tensor, name, torch.int32, (rows,))
-        pointer, stride = self._state_rows(state, offset, heads * dim * value_dim, "state")
+        columns = lib.lsa_delta_state_columns()
+        pointer, stride = self._state_rows(state, offset, heads * dim * (-(-value_dim // columns) * columns), "state")
+        if pointer % 16 or stride % 4:
+            raise ValueError("the delta rule's matrices start at multiples of 16 bytes in every slot")
         _launched(lib.lsa_delta_rule(_ptr(prepared), _ptr(strength), _ptr(decay), 1 if per_channel else 0, pointer, stride, _ptr(state_slots),
                                      _ptr(row_start), _ptr(row_len), _ptr(row_ctx), _ptr(out), rows, heads, kv_heads, dim, value_dim, _stream()),
                   "delta_rule")

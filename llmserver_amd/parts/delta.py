@@ -13,7 +13,8 @@ or a low-rank map of it (per head and key channel).  Each head's ``o`` is divide
 by a weight shared by the heads and by a gate (``silu`` of a projection, or ``sigmoid`` of a low-rank map), then the
 output projection.
 
-What a request keeps: the matrices ``[heads, dim, vdim]`` in float32 and, behind them, the last ``taps - 1`` inputs
+What a request keeps: the matrices in float32 (per head blocks of 16 value columns, ``[heads, vdim / 16, dim, 16]``, so
+that a workgroup's share is one contiguous piece) and, behind them, the last ``taps - 1`` inputs
 of the three convolutions, oldest first; zeros before a sequence's first token.  Everything behind the projections
 and convolutions (unit norms, softplus, exponentials, sigmoid of the write strength, state, read-out, per-head norm) is
 32-bit.
@@ -29,6 +30,12 @@ from .base import VECTOR, Mixer, ParamSpec, StateSpec
 from .linear import Linear
 
 UNIT_EPS = 1e-6         # q / sqrt(sum(q^2) + UNIT_EPS)
+STATE_COLUMNS = 16      # a head's matrix is kept as blocks of this many value columns, [vdim / 16][dim][16], the last one filled up
+
+
+def matrix_floats(heads: int, dim: int, value_dim: int) -> int:
+    """The size of a request's matrices as the kernels keep them."""
+    return heads * dim * (-(-value_dim // STATE_COLUMNS) * STATE_COLUMNS)
 
 
 @dataclasses.dataclass(frozen=True)
@@ -67,7 +74,7 @@ class GatedDeltaRule(Mixer):
         self.q_scale = float(dim) ** -0.5
         self.keys, self.values = kv_heads * dim, heads * value_dim
         self.channels = 2 * self.keys + self.values             # what the convolutions run over: q | k | v
-        self.matrix_size = heads * dim * value_dim
+        self.matrix_size = matrix_floats(heads, dim, value_dim)
         n = names
         # Everything that reads the mixer's input is one product: q | k | v | write strength | decay (or its inner
         # rows) | gate (or its inner rows).
@@ -87,7 +94,8 @@ class GatedDeltaRule(Mixer):
                 self.gate_low if self.low_rank_gate else self.values)
 
     def cache_spec(self):
-        return StateSpec((self.matrix_size + (self.taps - 1) * self.channels,), "float32")
+        # (a multiple of four numbers, so that every slot's matrices start at a multiple of 16 bytes)
+        return StateSpec((-(-(self.matrix_size + (self.taps - 1) * self.channels) // 4) * 4,), "float32")
 
     def param_specs(self):
         n = self.names

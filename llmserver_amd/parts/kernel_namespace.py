@@ -234,8 +234,8 @@ class KernelNamespace:
         """Per head ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` over each row's tokens, with
         ``prepared [T, C]``, ``strength [T, heads]`` (beta) and ``decay`` (g: ``[T, heads]``, or, ``per_channel``, ``[T, heads *
         dim]``, a decay for every row of ``S``) from :meth:`delta_prepare`; head ``h`` reads query/key head ``h // (heads /
-        kv_heads)``.  ``S [heads, dim, value_dim]`` float32 lives in ``state[slot, offset:]``, zeros before a sequence's first
-        token.  ``out [T, heads * value_dim]`` float32."""
+        kv_heads)``.  ``S`` lives in ``state[slot, offset:]`` in float32 as blocks of 16 value columns, ``[heads, ceil(value_dim /
+        16), dim, 16]``; zeros before a sequence's first token.  ``out [T, heads * value_dim]`` float32."""
         raise NotImplementedError
 
     # Routed experts.

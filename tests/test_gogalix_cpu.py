@@ -99,7 +99,8 @@ def test_the_model_declares_the_checkpoints_tensors_and_its_caches():
     caches = model.cache_specs()
     assert sorted(caches) == [0, 1, 2, 4]                    # the fourth layer reads the first one's pages
     assert caches[0] == PagedKVSpec(4, 16, 11)               # two maps of two key heads; kept for the longer of the two windows
-    assert caches[1] == StateSpec((4 * 8 * 6 + 2 * (16 + 16 + 24),), "float32") and caches[2] == StateSpec((2 * 12 * 5 + 3 * (12 + 12 + 10),), "float32")
+    # (a delta rule's matrices are kept in blocks of 16 value columns, the last one filled up)
+    assert caches[1] == StateSpec((4 * 8 * 16 + 2 * (16 + 16 + 24),), "float32") and caches[2] == StateSpec((2 * 12 * 16 + 3 * (12 + 12 + 10) + 2,), "float32")
     assert [(call.block, call.cache, call.writes_cache) for call in model.order] == [(0, 0, True), (1, 1, True), (2, 2, True), (3, 0, False), (4, 4, True)]
     assert not model.tie_head and not model.ignored_names()
     assert build_model(config_from_dict(dict(GB))).cache_specs()[2] == PagedKVSpec(2, 32, None)      # read through a window, kept for ever

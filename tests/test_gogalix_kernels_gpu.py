@@ -62,7 +62,7 @@ def _delta_step(which, dtype, sizes, taps, proj, extra, weights, state, slots, l
     token_row, positions, row_start, row_len, row_ctx = batch(lengths, firsts, "cuda")
     n = proj.shape[0]
     conv, scale, bias = weights
-    matrix = heads * dim * vdim
+    matrix = heads * dim * (-(-vdim // 16) * 16)
     prepared = torch.empty(n, channels, device="cuda")
     strengths = torch.empty(n, heads, device="cuda")
     decays = torch.empty(n, heads * dim if per_channel else heads, device="cuda")
@@ -89,8 +89,8 @@ def test_delta_rule_over_steps_and_slots(ops, dtype, per_channel, heads, kv_head
     twin = TorchOps()
     keys, values = kv_heads * dim, heads * vdim
     channels = 2 * keys + values
-    size = heads * dim * vdim + (taps - 1) * channels
-    states = [torch.randn(4, size + 3, device="cuda") for _ in range(2)]
+    size = heads * dim * (-(-vdim // 16) * 16) + (taps - 1) * channels
+    states = [torch.randn(4, -(-size // 4) * 4 + 4, device="cuda") for _ in range(2)]        # (slots start at multiples of 16 bytes)
     states[1].copy_(states[0])
     slots = torch.tensor([2, 0, 3], dtype=torch.int32, device="cuda")
     conv = torch.randn(channels, taps, device="cuda") * 0.6
@@ -116,7 +116,7 @@ def test_a_delta_rule_does_not_depend_on_how_its_tokens_are_cut(ops):
     """State and read-out are the same bits whether a sequence comes whole, in portions or token by token."""
     heads, kv_heads, dim, vdim, taps = 2, 1, 48, 20, 3
     channels = 2 * kv_heads * dim + heads * vdim
-    size = heads * dim * vdim + (taps - 1) * channels
+    size = heads * dim * (-(-vdim // 16) * 16) + (taps - 1) * channels
     conv, scale, bias = torch.randn(channels, taps, device="cuda") * 0.6, torch.randn(heads, device="cuda") * 0.5, torch.randn(heads, device="cuda")
     total = 45
     proj = torch.randn(total, channels + 2 * heads, device="cuda")

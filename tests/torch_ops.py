@@ -546,7 +546,8 @@ class TorchOps(KernelNamespace):
 
     def delta_rule(self, prepared, strength, decay, per_channel, state, offset, state_slots, row_start, row_len, row_ctx, out,
                    heads, kv_heads, dim, value_dim):
-        keys, size, repeat = kv_heads * dim, heads * dim * value_dim, heads // kv_heads
+        blocks = -(-value_dim // 16)
+        keys, size, repeat = kv_heads * dim, heads * dim * blocks * 16, heads // kv_heads
         beta = strength
         g = decay.view(-1, heads, dim)[..., None] if per_channel else decay[:, :, None, None]
         for row in range(len(row_len)):
@@ -554,7 +555,8 @@ class TorchOps(KernelNamespace):
             if count <= 0:
                 continue
             slot = int(state_slots[row])
-            matrix = state[slot, offset:offset + size].view(heads, dim, value_dim).clone()
+            # (kept as blocks of 16 value columns, [heads, blocks, dim, 16])
+            matrix = state[slot, offset:offset + size].view(heads, blocks, dim, 16).permute(0, 2, 1, 3).reshape(heads, dim, blocks * 16)[..., :value_dim].clone()
             if end - count == 0:
                 matrix.zero_()
             for t in range(start, start + count):
@@ -565,7 +567,9 @@ class TorchOps(KernelNamespace):
                 u = beta[t][:, None] * (v - torch.einsum("hdv,hd->hv", matrix, k))
                 matrix = matrix + k[:, :, None] * u[:, None, :]
                 out[t] = torch.einsum("hdv,hd->hv", matrix, q).reshape(-1)
-            state[slot, offset:offset + size] = matrix.reshape(-1)
+            kept = matrix.new_zeros((heads, dim, blocks * 16))           # (columns beyond the values are zeros)
+            kept[..., :value_dim] = matrix
+            state[slot, offset:offset + size] = kept.view(heads, dim, blocks, 16).permute(0, 2, 1, 3).reshape(-1)
 
     # -- routed experts ----------------------------------------------------------------------------------
     def route_experts(self, x, router, top, chosen, weights, scoring="softmax", groups=None, bias=None):
