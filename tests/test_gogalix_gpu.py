@@ -170,10 +170,28 @@ def test_greedy_generation_through_the_entry_point():
     assert same >= 0.6 * sum(len(e) for e in expected), (rounded, expected)
 
 
-def test_the_design_option_of_bench(tmp_path):
-    """``bench.py --design gogalix`` prints one JSON line with every named size beside its neighbours."""
+def test_the_benchmark_command_line_and_the_design_option_of_bench(tmp_path, capsys):
+    """The framework's command line serves a Gogalix folder like any other (matrix of prompt lengths and batch sizes, one
+    prompt's tokens equal to the oracle's; the mixed workload); ``bench.py --design gogalix`` prints one JSON line with
+    every named size beside its neighbours (three layers each here)."""
+    from llmserver_amd.cli import benchmark
+    print("command lines", flush=True)
+    folder, raw = model_folder("GC"), CASES["GC"][0]
+    report = tmp_path / "report.json"
+    assert benchmark.main(["--model", folder, "--dtype", "float32", "--prompt-tokens", "9,40", "--batch-sizes", "1,3", "--output-tokens", "6",
+                           "--repeats", "1", "--block-size", "16", "--json", str(report)]) == 0
+    results = json.loads(report.read_text())["results"]
+    assert [(r["prompt_tokens"], r["batch"]) for r in results] == [(9, 1), (9, 3), (40, 1), (40, 3)]
+    config, tensors = plain_model("GC")
+    prompt = benchmark.matrix_prompts(raw["vocab"], 9, 1, "whole-run", 0, 0)[0]
+    assert results[0]["tokens"][0] == plain.greedy_generate(config, tensors, prompt, 6)
+    capsys.readouterr()
+    assert benchmark.main(["--model", folder, "--mixed-requests", "6", "--mixed-prompt-range", "4,40", "--shared-prefix-tokens", "16",
+                           "--output-tokens", "5", "--block-size", "8", "--max-num-batched-tokens", "64"]) == 0
+    assert "mixed: 6 requests" in capsys.readouterr().out
     done = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--design", "gogalix", "--layers", "3", "--steps", "4", "--warmup", "1",
                            "--prefill-tokens", "256"], capture_output=True, text=True, timeout=600)
     assert done.returncode == 0, done.stderr[-3000:]
     record = json.loads([line for line in done.stdout.splitlines() if line.strip()][-1])
     assert set(record["sizes"]) == {"gogalix-2k", "barotar-2k", "dense-2k", "gogalix-4k", "barotar-4k", "dense-4k"} and record["value"] > 0
+    assert all(entry["layers"] == 3 and entry["decode_b8_tok_s"] > 0 and entry["prefill_256_ms"] > 0 for entry in record["sizes"].values())
