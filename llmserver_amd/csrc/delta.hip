@@ -272,11 +272,16 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
         if (tokens == CHUNK) {
             // a whole chunk runs unrolled: a token's LDS loads are issued ahead of the token before it, and its read-out's
             // sum across lanes overlaps the next token's walk
+            // (the read-outs wait in registers for the chunk's end: a store under a condition between two tokens would end
+            // the stretch of code that the loads can move within)
+            float r[CHUNK];
 #pragma unroll
-            for (int j = 0; j < CHUNK; ++j) {
-                const float r = delta_token<DP, PER_CHANNEL>(S, &s_k[j][p * DP], &s_q[j][p * DP], PER_CHANNEL ? &s_g[j][p * DP] : nullptr,
-                                                             PER_CHANNEL ? 1.f : s_decay[j], s_beta[j], s_v[j][local]);
-                if (writes) o[(size_t)j * heads * value_dim] = r;
+            for (int j = 0; j < CHUNK; ++j)
+                r[j] = delta_token<DP, PER_CHANNEL>(S, &s_k[j][p * DP], &s_q[j][p * DP], PER_CHANNEL ? &s_g[j][p * DP] : nullptr,
+                                                    PER_CHANNEL ? 1.f : s_decay[j], s_beta[j], s_v[j][local]);
+            if (writes) {
+#pragma unroll
+                for (int j = 0; j < CHUNK; ++j) o[(size_t)j * heads * value_dim] = r[j];
             }
         } else {
             for (int j = 0; j < tokens; ++j) {
