@@ -12,36 +12,73 @@ __device__ inline float softplus_of(float z) { return z > 20.f ? z : log1pf(expf
 
 // ---- a block whose sublayers' results join the stream together ---------------------------------------------------------
 // x[t] += s1 * sigmoid(gates[t][:W]) * y1[t] + s2 * sigmoid(gates[t][W:]) * y2[t] (y2 may be absent), in float32 where x
-// lies; then, with next_weight, normed[t] = x[t] * rsqrt(mean(x[t]^2) + eps) * next_weight.  One workgroup a token; a
-// thread keeps its columns in registers between the sum and the norm (rows of up to 256 * 4 * COLS numbers, longer ones
-// read the stored row again).
-template <typename G, typename Y1, typename Y2, typename N>
+// lies; then, with next_weight, normed[t] = x[t] * rsqrt(mean(x[t]^2) + eps) * next_weight.  One workgroup a token.  Rows of
+// up to 256 * COLS numbers (COLS > 0): a thread issues all its loads (the stream, gates, results, scales, the next norm's
+// weights) before the first store and before the sum of squares, so a row of one token waits for memory once, and keeps its
+// columns in registers between the sum and the norm.  Longer rows walk their columns and read the stored row again.
+constexpr int UPDATE_COLS = 16;
+template <typename G, typename Y1, typename Y2, typename N, int COLS>
 __global__ __launch_bounds__(256) void gated_pair_update_kernel(float* __restrict__ x, const G* __restrict__ gates, int gate_width,
                                                                 const Y1* __restrict__ y1, const float* __restrict__ s1,
                                                                 const Y2* __restrict__ y2, const float* __restrict__ s2,
                                                                 const float* __restrict__ next_weight, float eps, N* __restrict__ normed, int width) {
     __shared__ float scratch[16];
-    constexpr int COLS = 8;
     const int t = blockIdx.x;
     float* row = x + (size_t)t * width;
     const G* g = gates + (size_t)t * gate_width;
-    float kept[COLS];
+    if constexpr (COLS > 0) {
+        float xv[COLS > 0 ? COLS : 1], g1[COLS > 0 ? COLS : 1], a1[COLS > 0 ? COLS : 1], w1[COLS > 0 ? COLS : 1], g2[COLS > 0 ? COLS : 1],
+            a2[COLS > 0 ? COLS : 1], w2[COLS > 0 ? COLS : 1], nw[COLS > 0 ? COLS : 1];
+        // every load is of a place that is there (a column beyond the row reads the row's last one, an absent second
+        // sublayer reads the first one's operands, an absent norm the first scale), so none stands under a condition
+        // (the launcher makes Y2 float where there is no second sublayer, so the stream's own row can stand in)
+        const Y2* second = y2 ? y2 + (size_t)t * width : reinterpret_cast<const Y2*>(row);
+        const float* second_scale = y2 ? s2 : s1;
+        const float* following = next_weight ? next_weight : s1;
+        const int second_gate = y2 ? width : 0;
+        const float counts = y2 ? 1.f : 0.f;
+#pragma unroll
+        for (int n = 0; n < COLS; ++n) {
+            const int c = min((int)threadIdx.x + 256 * n, width - 1);
+            xv[n] = row[c];
+            g1[n] = (float)g[c];
+            a1[n] = (float)y1[(size_t)t * width + c];
+            w1[n] = s1[c];
+            g2[n] = (float)g[second_gate + c];
+            a2[n] = (float)second[c];
+            w2[n] = second_scale[c] * counts;
+            nw[n] = following[c];
+        }
+        float sq = 0.f;
+#pragma unroll
+        for (int n = 0; n < COLS; ++n) {
+            xv[n] += w1[n] * sigmoid_of(g1[n]) * a1[n] + w2[n] * sigmoid_of(g2[n]) * a2[n];
+            if ((int)threadIdx.x + 256 * n < width) sq += xv[n] * xv[n];
+        }
+#pragma unroll
+        for (int n = 0; n < COLS; ++n) {
+            const int c = threadIdx.x + 256 * n;
+            if (c < width) row[c] = xv[n];
+        }
+        if (!next_weight) return;
+        const float inv = rsqrtf(block_sum(sq, scratch) / (float)width + eps);
+#pragma unroll
+        for (int n = 0; n < COLS; ++n) {
+            const int c = threadIdx.x + 256 * n;
+            if (c < width) normed[(size_t)t * width + c] = (N)(xv[n] * inv * nw[n]);
+        }
+        return;
+    }
     float sq = 0.f;
-    int n = 0;
-    for (int c = threadIdx.x; c < width; c += 256, ++n) {
+    for (int c = threadIdx.x; c < width; c += 256) {
         float v = row[c] + s1[c] * sigmoid_of((float)g[c]) * (float)y1[(size_t)t * width + c];
         if (y2) v += s2[c] * sigmoid_of((float)g[width + c]) * (float)y2[(size_t)t * width + c];
         row[c] = v;
-        if (n < COLS) kept[n] = v;
         sq += v * v;
     }
     if (!next_weight) return;
     const float inv = rsqrtf(block_sum(sq, scratch) / (float)width + eps);
-    n = 0;
-    for (int c = threadIdx.x; c < width; c += 256, ++n) {
-        const float v = n < COLS ? kept[n] : row[c];
-        normed[(size_t)t * width + c] = (N)(v * inv * next_weight[c]);
-    }
+    for (int c = threadIdx.x; c < width; c += 256) normed[(size_t)t * width + c] = (N)(row[c] * inv * next_weight[c]);
 }
 
 // ---- differential attention: a1 - lambda a2 per head, divided by its root mean square, times a constant -------------------
@@ -110,11 +147,16 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(const T* __restrict__
     for (int e = lane; e < size; e += 64, ++n) {
         const int c = base + e;
         float acc = 0.f;
+        // both places a tap's input can come from are read, at rows that are there, and one is chosen: no load stands
+        // under a condition, so a thread's loads are in flight together
+        const float* kept_rows = mine ? mine : w;
+#pragma unroll 4
         for (int j = 0; j < taps; ++j) {
             const int back = kept - j, place = position - back;
-            if (place < 0) continue;
-            const float v = place >= first ? (float)proj[(size_t)(t - back) * stride + c] : mine[(size_t)(kept - (first - place)) * channels + c];
-            acc += w[(size_t)c * taps + j] * v;
+            const bool in_step = place >= first, from_state = !in_step && place >= 0;
+            const float here = (float)proj[(size_t)(in_step ? t - back : t) * stride + c];
+            const float before = kept_rows[(size_t)(from_state ? kept - (first - place) : 0) * channels + c];
+            acc += w[(size_t)c * taps + j] * (in_step ? here : from_state ? before : 0.f);
         }
         acc *= sigmoid_of(acc);
         if (unit) {
@@ -309,8 +351,11 @@ LSA_EXPORT int lsa_gated_pair_update(float* x, const void* gates, int gates_code
                                      int normed_code, int n, int width, hipStream_t stream) {
     if (n <= 0) return 0;
     if (gate_width != (y2 ? 2 * width : width) || (y2 && !s2) || (next_weight && !normed)) return -1;
-#define LSA_LAUNCH(G, Y1, Y2, N) gated_pair_update_kernel<G, Y1, Y2, N><<<n, 256, 0, stream>>>(x, (const G*)gates, gate_width, (const Y1*)y1, s1, \
+    if (!y2) y2_code = 0;
+#define LSA_LAUNCH_R(G, Y1, Y2, N, R) gated_pair_update_kernel<G, Y1, Y2, N, R><<<n, 256, 0, stream>>>(x, (const G*)gates, gate_width, (const Y1*)y1, s1, \
         (const Y2*)y2, s2, next_weight, eps, (N*)normed, width)
+#define LSA_LAUNCH(G, Y1, Y2, N) do { if (width <= 1024) LSA_LAUNCH_R(G, Y1, Y2, N, 4); else if (width <= 2048) LSA_LAUNCH_R(G, Y1, Y2, N, 8); \
+                                      else if (width <= 256 * UPDATE_COLS) LSA_LAUNCH_R(G, Y1, Y2, N, UPDATE_COLS); else LSA_LAUNCH_R(G, Y1, Y2, N, 0); } while (0)
 #define LSA_BY_N(G, Y1, Y2) do { if (normed_code) LSA_LAUNCH(G, Y1, Y2, bf16_t); else LSA_LAUNCH(G, Y1, Y2, float); } while (0)
 #define LSA_BY_Y2(G, Y1) do { if (y2_code) LSA_BY_N(G, Y1, bf16_t); else LSA_BY_N(G, Y1, float); } while (0)
 #define LSA_BY_Y1(G) do { if (y1_code) LSA_BY_Y2(G, bf16_t); else LSA_BY_Y2(G, float); } while (0)
@@ -319,6 +364,7 @@ LSA_EXPORT int lsa_gated_pair_update(float* x, const void* gates, int gates_code
 #undef LSA_BY_Y2
 #undef LSA_BY_N
 #undef LSA_LAUNCH
+#undef LSA_LAUNCH_R
     LSA_LAUNCH_CHECK();
 }
 
