@@ -20,7 +20,7 @@ def ops():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width", [8, 100, 256, 1027, 4400])
+@pytest.mark.parametrize("width", [8, 100, 320, 1027, 2048, 4400])
 @pytest.mark.parametrize("second", [None, torch.float32, "same"])
 def test_gated_pair_update(ops, dtype, width, second):
     print(f"gated_pair_update {dtype} {width} {second}", flush=True)
@@ -43,7 +43,7 @@ def test_gated_pair_update(ops, dtype, width, second):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("kv_heads,group,vdim,row", [(2, 3, 40, 48), (1, 1, 96, 96), (3, 2, 7, 16), (2, 1, 130, 144)])
+@pytest.mark.parametrize("kv_heads,group,vdim,row", [(2, 3, 40, 48), (1, 1, 80, 80), (3, 2, 7, 16), (2, 1, 130, 144)])
 def test_differential_heads(ops, dtype, kv_heads, group, vdim, row):
     print(f"differential_heads {dtype} {kv_heads} {group} {vdim} {row}", flush=True)
     twin = TorchOps()
@@ -81,7 +81,7 @@ def _delta_step(which, dtype, sizes, taps, proj, extra, weights, state, slots, l
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("per_channel", [False, True])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,taps", [(3, 3, 24, 40, 3), (4, 2, 64, 64, 4), (2, 1, 7, 100, 2), (1, 1, 130, 9, 1),
-                                                          (2, 2, 256, 17, 3), (6, 3, 32, 32, 5), (2, 2, 128, 128, 4)])
+                                                          (2, 2, 256, 17, 3), (6, 3, 24, 48, 5), (2, 2, 128, 128, 4)])
 def test_delta_rule_over_steps_and_slots(ops, dtype, per_channel, heads, kv_heads, dim, vdim, taps):
     """Rows of unequal portions, an empty row, single tokens, portions longer than the kernel's chunks and shorter than
     the convolution's reach; a request that starts again in a used slot starts from zeros."""
@@ -135,7 +135,7 @@ def test_a_delta_rule_does_not_depend_on_how_its_tokens_are_cut(ops):
         assert torch.equal(out, kept[0][0]) and torch.equal(state, kept[0][1])
 
 
-@pytest.mark.parametrize("experts,top", [(16, 3), (5, 5), (130, 2)])
+@pytest.mark.parametrize("experts,top", [(12, 4), (5, 5), (130, 2)])
 def test_a_router_with_a_bias(ops, experts, top):
     twin = TorchOps()
     for n in (3, 70):
